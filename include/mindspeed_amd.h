@@ -1,0 +1,188 @@
+/*
+ * mindspeed_amd.h — C ABI of the MI355X (gfx950) MoE expert hot path.
+ *
+ * One shared library, libmindspeed_amd.so, exports these entry points.  They
+ * take plain pointers, sizes and strides; every pointer is a device pointer
+ * unless stated otherwise.  Conventions shared by all entry points:
+ *
+ *   - return 0 (MS_OK) on success, a non-zero ms_status otherwise; the text of
+ *     the last failure on the calling thread is returned by ms_last_error();
+ *   - all work is enqueued on the given stream (a hipStream_t passed as
+ *     void*; NULL is the default stream); no entry point synchronises, reads
+ *     device data on the host, allocates or frees device memory;
+ *   - the caller owns inputs, outputs and workspace and keeps them alive until
+ *     the stream has passed the call; workspace sizes come from the matching
+ *     *_workspace_size function and may be over-provisioned;
+ *   - strides are in elements; row data of 16-bit types is processed with
+ *     16-byte vectors when pointers and strides allow it and with an
+ *     element-wise path otherwise (same results).
+ *
+ * Each declaration cites the reference interface (paths relative to the
+ * reference root) that it stands in for.  The reference reaches its vendor
+ * kernels through a two-phase "GetWorkspaceSize / run on stream" C ABI
+ * (mindspeed/ops/csrc/cann/inc/aclnn_common.h:587-644); this header keeps that
+ * two-phase shape.
+ */
+#ifndef MINDSPEED_AMD_H_
+#define MINDSPEED_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *ms_stream_t; /* hipStream_t */
+
+typedef enum ms_status {
+    MS_OK = 0,
+    MS_ERR_INVALID_ARGUMENT = 1,
+    MS_ERR_UNSUPPORTED = 2,
+    MS_ERR_WORKSPACE_TOO_SMALL = 3,
+    MS_ERR_HIP = 4
+} ms_status;
+
+typedef enum ms_dtype { MS_BF16 = 0, MS_FP16 = 1, MS_FP32 = 2 } ms_dtype;
+typedef enum ms_index_dtype { MS_INT32 = 0, MS_INT64 = 1 } ms_index_dtype;
+
+/* Largest expert id + 1 the permute sort accepts.  Ids outside [0, limit) are
+ * clamped into range for memory safety; results are then unspecified. */
+#define MS_MAX_EXPERTS 1024
+
+/* Library identification and error text (thread-local, never NULL). */
+int ms_version(void);
+const char *ms_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * Token permute — stands in for aclnnMoeTokenPermute as called from
+ * mindspeed/ops/csrc/cann/npu_moe_token_permute.cpp:65-97 (Python surface
+ * mindspeed/ops/npu_moe_token_permute.py:13-20).
+ *
+ * indices [num_tokens, topk] (int32 or int64 expert ids) are flattened
+ * token-major and stably sorted by expert id.  Outputs:
+ *   permuted_tokens [num_out_tokens, hidden]   row r = tokens[sorted_indices[r] / topk]
+ *   row_id_map      int32 [num_tokens*topk]    output row of flat position i
+ *                                              (entries >= num_out_tokens are dropped rows)
+ *   sorted_indices  int32 [num_out_tokens]     optional (may be NULL): flat position of row r,
+ *                                              the order the torch path returns
+ *                                              (mindspeed/core/transformer/moe/moe_utils.py:206-208)
+ *   tokens_per_expert int64 [num_experts_hint] optional (may be NULL; needs num_experts_hint > 0)
+ * num_experts_hint: number of experts if known (bounds the sort's key range),
+ * 0 if unknown (MS_MAX_EXPERTS is assumed).
+ * ---------------------------------------------------------------------- */
+int ms_moe_token_permute_workspace_size(int64_t num_tokens, int64_t topk,
+                                        int64_t num_experts_hint, size_t *bytes);
+int ms_moe_token_permute(ms_stream_t stream, const void *tokens, const void *indices,
+                         int index_dtype, int64_t num_tokens, int64_t topk, int64_t hidden,
+                         int dtype, int64_t num_out_tokens, int64_t num_experts_hint,
+                         void *permuted_tokens, int32_t *row_id_map, int32_t *sorted_indices,
+                         int64_t *tokens_per_expert, void *workspace, size_t workspace_bytes);
+
+/* Token permute backward — stands in for aclnnMoeTokenPermuteGrad
+ * (npu_moe_token_permute.cpp:99-118):
+ *   grad_tokens[t] = sum_j grad_permuted[row_id_map[t*topk+j]]  (dropped rows add 0),
+ * accumulated in fp32 and rounded once. */
+int ms_moe_token_permute_grad(ms_stream_t stream, const void *grad_permuted_tokens,
+                              const int32_t *row_id_map, int64_t num_tokens, int64_t topk,
+                              int64_t hidden, int dtype, int64_t num_permuted_rows,
+                              void *grad_tokens);
+
+/* Token unpermute — stands in for aclnnMoeTokenUnpermute
+ * (mindspeed/ops/csrc/cann/npu_moe_token_unpermute.cpp:95-122; Python surface
+ * mindspeed/ops/npu_moe_token_unpermute.py:13-22):
+ *   out[t] = sum_j probs[t,j] * permuted[row_id_map[t*topk+j]]
+ * probs may be NULL (unweighted sum).  fp32 accumulation, one rounding. */
+int ms_moe_token_unpermute(ms_stream_t stream, const void *permuted_tokens,
+                           const int32_t *row_id_map, const void *probs, int64_t num_tokens,
+                           int64_t topk, int64_t hidden, int dtype, int64_t num_permuted_rows,
+                           void *unpermuted_tokens);
+
+/* Token unpermute backward — stands in for aclnnMoeTokenUnpermuteGrad
+ * (npu_moe_token_unpermute.cpp:124-148):
+ *   grad_permuted[row_id_map[t*topk+j]] = probs[t,j] * grad_out[t]
+ *   grad_probs[t,j] = <grad_out[t], permuted[row_id_map[t*topk+j]]>   (fp32 dot)
+ * probs / grad_probs / permuted_tokens may be NULL together (then
+ * grad_permuted[row] = grad_out[token of row]). */
+int ms_moe_token_unpermute_grad(ms_stream_t stream, const void *permuted_tokens,
+                                const void *grad_unpermuted_tokens, const int32_t *row_id_map,
+                                const void *probs, int64_t num_tokens, int64_t topk,
+                                int64_t hidden, int dtype, int64_t num_permuted_rows,
+                                void *grad_permuted_tokens, void *grad_probs);
+
+/* ------------------------------------------------------------------------
+ * Grouped matmul — stands in for aclnnGroupedMatmulV2 / V4 as called from
+ * mindspeed/ops/csrc/cann/gmm.cpp:77-167 (Python surface
+ * mindspeed/ops/gmm.py:164-175), including the backward recipes of
+ * gmm.cpp:169-246 which are further calls of the same entry point on
+ * transposed views, and, with accumulate != 0, for the ATB
+ * GroupedMatmulInplaceAdd call of
+ * mindspeed/ops/csrc/atb/groupmatmul_add.cpp:39-64.
+ *
+ * group_type 0 (split on rows of x):
+ *     x [m, k], weight [num_groups, k, n], y [m, n];
+ *     y[o_g:o_{g+1}] = x[o_g:o_{g+1}] @ weight[g]; rows past the last offset are zero.
+ * group_type 2 (split on the reduction dim):
+ *     x [k, m] (normally a transposed view), weight [m, n], y [num_groups, k, n];
+ *     y[g] = x[:, o_g:o_{g+1}] @ weight[o_g:o_{g+1}]; an empty group gives zeros.
+ * group_list: device int64 [num_groups]; group_list_type 0 = cumulative
+ * offsets (npu_gmm), 1 = per-group counts (npu_gmm_v2).  It is never read on
+ * the host.
+ * x / weight are addressed through explicit element strides, so transposed
+ * views need no copy; for each of x and weight one of the two matrix strides
+ * must be 1.  y is row-major with row stride y_stride_row (group_type 2:
+ * group stride k*y_stride_row).
+ * dtype: element type of x and weight (bf16 / fp16: MFMA 32x32x16 with fp32
+ * accumulation; fp32: MFMA 32x32x2 fp32).  out_dtype: dtype, or MS_FP32.
+ * accumulate != 0: y += result (requires out_dtype == MS_FP32).
+ * ---------------------------------------------------------------------- */
+int ms_gmm_workspace_size(int64_t num_groups, int64_t m, int group_type, size_t *bytes);
+int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1,
+           const void *weight, int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1,
+           void *y, int64_t y_stride_row, const int64_t *group_list, int group_list_type,
+           int group_type, int64_t num_groups, int64_t m, int64_t k, int64_t n, int dtype,
+           int out_dtype, int accumulate, void *workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
+ * SwiGLU (+ optional per-row probability) — stands in for the ATB
+ * ACTIVATION_SWIGLU_FORWARD / BACKWARD calls of
+ * mindspeed/ops/csrc/atb/swiglu.cpp:64-126 and the probs product of
+ * mindspeed/core/transformer/moe/moe_feature/gmm/experts.py:41-44:
+ *   y[r, c] = silu(x[r, c]) * x[r, ffn + c] * (probs ? probs[r] : 1)
+ * x [rows, 2*ffn], y [rows, ffn], probs fp32-or-dtype [rows] (probs_dtype).
+ * Backward writes grad_x [rows, 2*ffn] and, if probs, grad_probs [rows]
+ * (same dtype as probs). fp32 math, one rounding.
+ * ---------------------------------------------------------------------- */
+int ms_swiglu(ms_stream_t stream, const void *x, const void *probs, int probs_dtype,
+              int64_t rows, int64_t ffn, int dtype, void *y);
+int ms_swiglu_grad(ms_stream_t stream, const void *grad_y, const void *x, const void *probs,
+                   int probs_dtype, int64_t rows, int64_t ffn, int dtype, void *grad_x,
+                   void *grad_probs);
+
+/* ------------------------------------------------------------------------
+ * Chunk sort — stands in for sort_chunks_by_idxs of the alltoall dispatcher
+ * (torch statement: mindspeed/core/transformer/moe/moe_feature/overlap/
+ * moe_common.py:377-398; fused form: mindspeed/lite/ops/triton/
+ * sort_chunks_by_idx.py:300-348):
+ *   out = cat([split(input, split_sizes)[i] for i in sorted_idxs])
+ * split_sizes int64 [num_chunks] and sorted_idxs int64 [num_chunks] are device
+ * arrays.  row_map int32 [rows] receives the source row of every output row
+ * (the backward is the same call with the inverse map, see ms_gather_rows).
+ * probs (optional, [rows], probs_dtype) are reordered into out_probs.
+ * ---------------------------------------------------------------------- */
+int ms_sort_chunks(ms_stream_t stream, const void *input, const int64_t *split_sizes,
+                   const int64_t *sorted_idxs, int64_t num_chunks, int64_t rows, int64_t hidden,
+                   int dtype, const void *probs, int probs_dtype, void *out, void *out_probs,
+                   int32_t *row_map);
+/* out[r] = input[row_map[r]] (inverse != 0: out[row_map[r]] = input[r]). */
+int ms_gather_rows(ms_stream_t stream, const void *input, const int32_t *row_map, int64_t rows,
+                   int64_t hidden, int dtype, int inverse, void *out);
+
+/* Plain device copy kernel (16-byte vectors, grid-stride).  Used to calibrate
+ * profiler byte counters against a transfer of known size. */
+int ms_copy_bytes(ms_stream_t stream, const void *src, void *dst, size_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MINDSPEED_AMD_H_ */

@@ -1,0 +1,68 @@
+"""Build recipe for libmindspeed_amd.so (hipcc, gfx950 only, in-tree).
+
+``python -m mindspeed_amd.build`` compiles every ``csrc/*.hip`` translation
+unit for gfx950 and links them into ``mindspeed_amd/libmindspeed_amd.so``.
+hipcc cross-compiles, so this works on a host without a GPU.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ_DIR = os.path.join(HERE, "build")
+LIB_PATH = os.path.join(HERE, "libmindspeed_amd.so")
+
+ARCH = "gfx950"
+# packed-fp32 VALU forms are switched off for every device translation unit.
+HIPCC_FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: the MI355X kernels cannot be built")
+    return exe
+
+
+def sources():
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def _compile(src: str, force: bool) -> str:
+    obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
+    deps = [src, os.path.join(CSRC, "common.h"), os.path.join(HERE, "..", "include", "mindspeed_amd.h")]
+    if not force and os.path.exists(obj) and all(os.path.getmtime(obj) > os.path.getmtime(d) for d in deps):
+        return obj
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", src, "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src}:\n{res.stderr}")
+    return obj
+
+
+def build(force: bool = True, verbose: bool = False) -> str:
+    """Compile and link the library; returns its path."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    srcs = sources()
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        objs = list(pool.map(lambda s: _compile(s, force), srcs))
+    cmd = [_hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stderr}")
+    if verbose:
+        print(f"built {LIB_PATH} from {len(srcs)} translation units")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build(force="--incremental" not in sys.argv, verbose=True)

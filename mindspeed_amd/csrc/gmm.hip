@@ -1,0 +1,605 @@
+// Grouped matmul for gfx950 (MI355X): y[rows of group g] = x[rows of g] @ w[g]
+// (split on rows) and y[g] = x[:, red range of g] @ w[red range of g] (split on
+// the reduction dim), for forward, dX and dW from one weight storage.
+//
+// Structure
+//   * gmm_schedule_kernel turns the device-resident group_list into a table of
+//     per-group tile ranges (no host read of group_list, empty groups emit no
+//     row tiles, a trailing pseudo-group zero-fills rows past the last offset).
+//   * gmm16_kernel: bf16 / fp16, 256x256x64 macro tile per 256-thread workgroup
+//     (2x2 wavefronts, 128x128 per wavefront = 4x4 v_mfma_f32_32x32x16), fp32
+//     accumulators, LDS double buffer (128 KB of the CU's 160 KB), operands
+//     stored in LDS as [outer][reduction] with an XOR swizzle of the 16-byte
+//     chunks so ds_read_b128 fragment loads are bank-conflict free.  Operands
+//     whose contiguous memory dim is not the reduction dim are transposed in
+//     registers (8x8 blocks) on their way from global memory to LDS, so NN, NT
+//     and TN products all run the same inner loop.
+//   * tiles are rasterised per XCD: workgroup b runs on XCD b%8, each XCD owns a
+//     contiguous range of logical tiles ordered row-tile-fastest inside a column
+//     panel, so concurrently running workgroups of an XCD share weight panels
+//     in that XCD's L2.
+//   * gmm32_kernel: fp32 inputs, v_mfma_f32_32x32x2f32, 128x128x8 tiles.
+#include "common.h"
+
+namespace ms {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kMaxGroups = 4096;
+
+struct GroupEntry {
+    int row_begin, row_end;  // output rows of the group
+    int red_begin, red_end;  // reduction range of the group
+    int tile_begin;          // first logical tile
+    int num_row_tiles;
+    int64_t b_off;           // element offset of the group's weight block
+    int64_t c_off;           // element offset of the group's output block
+};
+
+struct TileTable {
+    int total_tiles;
+    int num_entries;
+    int pad[6];
+    GroupEntry entries[1];
+};
+
+struct GmmArgs {
+    const void *a;
+    const void *b;
+    void *c;
+    const TileTable *table;
+    int64_t a_stride_row, a_stride_red;
+    int64_t b_stride_red, b_stride_col;
+    int64_t c_stride_row;
+    int cols;          // n
+    int num_col_tiles;
+    int a_vec_ok, b_vec_ok, c_vec_ok;
+};
+
+// ---- schedule ------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__restrict__ group_list,
+                                                           int group_list_type, int group_type, int num_groups,
+                                                           int m, int k, int tile_rows, int num_col_tiles,
+                                                           int64_t b_stride_group, int64_t c_stride_group,
+                                                           TileTable *table) {
+    extern __shared__ int64_t gl[];
+    for (int g = threadIdx.x; g < num_groups; g += blockDim.x) gl[g] = group_list[g];
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    int64_t prev = 0;
+    int tiles = 0;
+    int n = 0;
+    for (int g = 0; g < num_groups; ++g) {
+        int64_t end = group_list_type == 0 ? gl[g] : prev + gl[g];
+        end = end < prev ? prev : end;
+        end = end > m ? m : end;
+        GroupEntry e;
+        if (group_type == 0) {
+            e.row_begin = static_cast<int>(prev);
+            e.row_end = static_cast<int>(end);
+            e.red_begin = 0;
+            e.red_end = k;
+            e.b_off = g * b_stride_group;
+            e.c_off = 0;
+        } else {
+            e.row_begin = 0;
+            e.row_end = k;
+            e.red_begin = static_cast<int>(prev);
+            e.red_end = static_cast<int>(end);
+            e.b_off = 0;
+            e.c_off = g * c_stride_group;
+        }
+        e.num_row_tiles = (e.row_end - e.row_begin + tile_rows - 1) / tile_rows;
+        e.tile_begin = tiles;
+        tiles += e.num_row_tiles * num_col_tiles;
+        table->entries[n++] = e;
+        prev = end;
+    }
+    if (group_type == 0 && prev < m) {  // rows past the last offset: zero-fill
+        GroupEntry e;
+        e.row_begin = static_cast<int>(prev);
+        e.row_end = m;
+        e.red_begin = 0;
+        e.red_end = 0;
+        e.b_off = 0;
+        e.c_off = 0;
+        e.num_row_tiles = (e.row_end - e.row_begin + tile_rows - 1) / tile_rows;
+        e.tile_begin = tiles;
+        tiles += e.num_row_tiles * num_col_tiles;
+        table->entries[n++] = e;
+    }
+    table->total_tiles = tiles;
+    table->num_entries = n;
+}
+
+struct TileCoord {
+    GroupEntry e;
+    int row_tile, col_tile;
+    bool valid;
+};
+
+// Map this workgroup to its logical tile (XCD-aware, see file header).
+__device__ __forceinline__ TileCoord locate_tile(const TileTable *table) {
+    TileCoord tc;
+    tc.valid = false;
+    const int total = table->total_tiles;
+    const int per_xcd = (total + 7) >> 3;
+    const int xcd = blockIdx.x & 7;
+    const int slot = blockIdx.x >> 3;
+    if (slot >= per_xcd) return tc;
+    const int logical = xcd * per_xcd + slot;
+    if (logical >= total) return tc;
+    int lo = 0, hi = table->num_entries;  // last entry with tile_begin <= logical
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (table->entries[mid].tile_begin <= logical) lo = mid; else hi = mid;
+    }
+    tc.e = table->entries[lo];
+    const int r = logical - tc.e.tile_begin;
+    tc.col_tile = r / tc.e.num_row_tiles;
+    tc.row_tile = r - tc.col_tile * tc.e.num_row_tiles;
+    tc.valid = true;
+    return tc;
+}
+
+// ---- 16-bit MFMA kernel ------------------------------------------------------------------
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int kTileBytes = BM * BK * 2;                 // 32 KB per operand per stage
+constexpr int kLdsBytes16 = 4 * kTileBytes;             // A,B x 2 stages = 128 KB
+
+enum OutMode { OUT_SAME = 0, OUT_F32 = 1, ACC_F32 = 2 };
+
+template <int DT>
+__device__ __forceinline__ f32x16 mfma16(v16 a, v16 b, f32x16 c) {
+    if constexpr (DT == MS_BF16) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                       0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                      0, 0);
+    }
+}
+
+// 8 contiguous 16-bit elements starting at p; elements >= nvalid read as zero.
+__device__ __forceinline__ v16 load8(const uint16_t *p, int nvalid, bool vec_ok) {
+    if (nvalid >= 8 && vec_ok && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) return *reinterpret_cast<const v16 *>(p);
+    v16 r = {0u, 0u, 0u, 0u};
+    if (nvalid > 0) {
+        uint16_t tmp[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) tmp[e] = e < nvalid ? p[e] : static_cast<uint16_t>(0);
+        r = *reinterpret_cast<v16 *>(tmp);
+    }
+    return r;
+}
+
+// LDS swizzle: 16-byte chunk position of (row, chunk) inside the row's 128 bytes.
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// Operand tile loader.  RED == true: memory is contiguous along the reduction
+// dim; RED == false: contiguous along the outer (row of A / col of B) dim.
+template <bool RED>
+struct TileLoader {
+    v16 r[8];
+
+    // outer0/outer_end: first outer index of the tile and the exclusive bound of
+    // valid outer indices; red0/red_end likewise for this 64-wide reduction step.
+    __device__ __forceinline__ void load(const uint16_t *base, int64_t stride_outer, int64_t stride_red, int outer0,
+                                         int outer_end, int red0, int red_end, bool vec_ok) {
+        const int tid = threadIdx.x;
+        if constexpr (RED) {
+            const int ck = tid & 7;
+            const int red = red0 + ck * 8;
+            const int nvalid = red_end - red;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int outer = outer0 + (tid >> 3) + 32 * i;
+                const bool ok = outer < outer_end;
+                const uint16_t *p = base + static_cast<int64_t>(ok ? outer : outer0) * stride_outer + red;
+                r[i] = load8(p, ok ? nvalid : 0, vec_ok);
+            }
+        } else {
+            const int kb = tid & 7;
+            const int nb = tid >> 3;
+            const int outer = outer0 + nb * 8;
+            const int nvalid = outer_end - outer;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int red = red0 + kb * 8 + j;
+                const bool ok = red < red_end;
+                const uint16_t *p = base + static_cast<int64_t>(ok ? red : red0) * stride_red + outer;
+                r[j] = load8(p, ok ? nvalid : 0, vec_ok);
+            }
+        }
+    }
+
+    __device__ __forceinline__ void store(char *lds_tile) const {
+        const int tid = threadIdx.x;
+        if constexpr (RED) {
+            const int ck = tid & 7;
+            const int row = tid >> 3;
+            char *dst = lds_tile + row * 128 + ((ck ^ swz(row)) << 4);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) *reinterpret_cast<v16 *>(dst + i * 32 * 128) = r[i];
+        } else {
+            const int kb = tid & 7;
+            const int nb = tid >> 3;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                v16 o;
+#pragma unroll
+                for (int mth = 0; mth < 4; ++mth) {
+                    const unsigned lo = r[2 * mth][c >> 1];
+                    const unsigned hi = r[2 * mth + 1][c >> 1];
+                    o[mth] = (c & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+                }
+                const int row = nb * 8 + c;
+                *reinterpret_cast<v16 *>(lds_tile + row * 128 + ((kb ^ swz(row)) << 4)) = o;
+            }
+        }
+    }
+};
+
+template <int DT, bool A_RED, bool B_RED, int OUT>
+__global__ __launch_bounds__(256) void gmm16_kernel(const GmmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const TileCoord tc = locate_tile(p.table);
+    if (!tc.valid) return;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    const int row0 = tc.e.row_begin + tc.row_tile * BM;
+    const int row_end = tc.e.row_end;
+    const int col0 = tc.col_tile * BN;
+    const int col_end = p.cols;
+    const int red_begin = tc.e.red_begin, red_end = tc.e.red_end;
+
+    const uint16_t *a_base = static_cast<const uint16_t *>(p.a);
+    const uint16_t *b_base = static_cast<const uint16_t *>(p.b) + tc.e.b_off;
+    const bool a_vec = p.a_vec_ok != 0, b_vec = p.b_vec_ok != 0;
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    // per-lane fragment read offsets (bytes) inside an operand tile
+    const int frow = lane & 31;
+    const int fsw = swz(frow);
+    const int hi = lane >> 5;
+    int a_off[4], b_off[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+        const int chunk = ((kk * 2 + hi) ^ fsw) << 4;
+        a_off[kk] = (wm * 128 + frow) * 128 + chunk;
+        b_off[kk] = (wn * 128 + frow) * 128 + chunk;
+    }
+
+    TileLoader<A_RED> la;
+    TileLoader<B_RED> lb;
+    const int nk = (red_end - red_begin + BK - 1) / BK;
+    if (nk > 0) {
+        la.load(a_base, p.a_stride_row, p.a_stride_red, row0, row_end, red_begin, red_end, a_vec);
+        lb.load(b_base, p.b_stride_col, p.b_stride_red, col0, col_end, red_begin, red_end, b_vec);
+        la.store(lds);
+        lb.store(lds + kTileBytes);
+        __syncthreads();
+    }
+    for (int kt = 0; kt < nk; ++kt) {
+        char *sa = lds + (kt & 1) * 2 * kTileBytes;
+        char *sb = sa + kTileBytes;
+        const bool more = kt + 1 < nk;
+        if (more) {
+            const int red0 = red_begin + (kt + 1) * BK;
+            la.load(a_base, p.a_stride_row, p.a_stride_red, row0, row_end, red0, red_end, a_vec);
+            lb.load(b_base, p.b_stride_col, p.b_stride_red, col0, col_end, red0, red_end, b_vec);
+        }
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            v16 af[4], bf[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                af[t] = *reinterpret_cast<const v16 *>(sa + a_off[kk] + t * 32 * 128);
+                bf[t] = *reinterpret_cast<const v16 *>(sb + b_off[kk] + t * 32 * 128);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = mfma16<DT>(bf[j], af[i], acc[i][j]);
+        }
+        if (more) {
+            char *na = lds + ((kt + 1) & 1) * 2 * kTileBytes;
+            la.store(na);
+            lb.store(na + kTileBytes);
+        }
+        __syncthreads();
+    }
+
+    // Epilogue.  acc[i][j][4*q+e] = C[row0 + wm*128 + i*32 + (lane&31)]
+    //                                [col0 + wn*128 + j*32 + 8*q + 4*(lane>>5) + e]
+    const int64_t ldc = p.c_stride_row;
+    const bool c_vec = p.c_vec_ok != 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = row0 + wm * 128 + i * 32 + (lane & 31);
+        if (row >= row_end) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int col = col0 + wn * 128 + j * 32 + 8 * q + 4 * hi;
+                if (col >= col_end) continue;
+                const int64_t at = tc.e.c_off + static_cast<int64_t>(row) * ldc + col;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
+                const bool full = c_vec && col + 4 <= col_end;
+                if constexpr (OUT == OUT_SAME) {
+                    uint16_t *c = static_cast<uint16_t *>(p.c) + at;
+                    const bool full8 = full && (reinterpret_cast<uintptr_t>(c) & 7u) == 0;
+                    uint16_t h[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) h[e] = DT == MS_BF16 ? BF16::from_float(v[e]) : FP16::from_float(v[e]);
+                    if (full8) {
+                        *reinterpret_cast<uint2 *>(c) = *reinterpret_cast<uint2 *>(h);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (col + e < col_end) c[e] = h[e];
+                    }
+                } else {
+                    float *c = static_cast<float *>(p.c) + at;
+                    if (full && (reinterpret_cast<uintptr_t>(c) & 15u) == 0) {
+                        f32x4 o = {v[0], v[1], v[2], v[3]};
+                        if constexpr (OUT == ACC_F32) o += *reinterpret_cast<f32x4 *>(c);
+                        *reinterpret_cast<f32x4 *>(c) = o;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (col + e < col_end) c[e] = (OUT == ACC_F32 ? c[e] : 0.f) + v[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---- fp32 MFMA kernel ---------------------------------------------------------------------
+constexpr int FM = 128, FN = 128, FK = 8, FPITCH = 132;
+
+template <bool ACC>
+__global__ __launch_bounds__(256) void gmm32_kernel(const GmmArgs p) {
+    __shared__ float sa[FK][FPITCH];
+    __shared__ float sb[FK][FPITCH];
+    const TileCoord tc = locate_tile(p.table);
+    if (!tc.valid) return;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int row0 = tc.e.row_begin + tc.row_tile * FM;
+    const int row_end = tc.e.row_end;
+    const int col0 = tc.col_tile * FN;
+    const int col_end = p.cols;
+    const float *a_base = static_cast<const float *>(p.a);
+    const float *b_base = static_cast<const float *>(p.b) + tc.e.b_off;
+    const bool a_red = p.a_stride_red == 1, b_red = p.b_stride_red == 1;
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    for (int red0 = tc.e.red_begin; red0 < tc.e.red_end; red0 += FK) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int idx = tid + i * 256;
+            {
+                const int kk = a_red ? (idx & 7) : (idx >> 7);
+                const int r = a_red ? (idx >> 3) : (idx & 127);
+                const int row = row0 + r, red = red0 + kk;
+                sa[kk][r] = (row < row_end && red < tc.e.red_end)
+                                ? a_base[static_cast<int64_t>(row) * p.a_stride_row + static_cast<int64_t>(red) * p.a_stride_red]
+                                : 0.f;
+            }
+            {
+                const int kk = b_red ? (idx & 7) : (idx >> 7);
+                const int cc = b_red ? (idx >> 3) : (idx & 127);
+                const int col = col0 + cc, red = red0 + kk;
+                sb[kk][cc] = (col < col_end && red < tc.e.red_end)
+                                 ? b_base[static_cast<int64_t>(red) * p.b_stride_red + static_cast<int64_t>(col) * p.b_stride_col]
+                                 : 0.f;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < FK / 2; ++ks) {
+            const int kk = ks * 2 + (lane >> 5);
+            float av[2], bv[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                av[t] = sa[kk][wm * 64 + t * 32 + (lane & 31)];
+                bv[t] = sb[kk][wn * 64 + t * 32 + (lane & 31)];
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+    float *c_base = static_cast<float *>(p.c) + tc.e.c_off;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int row = row0 + wm * 64 + i * 32 + (lane & 31);
+        if (row >= row_end) continue;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int col = col0 + wn * 64 + j * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                if (col < col_end) {
+                    float *c = c_base + static_cast<int64_t>(row) * p.c_stride_row + col;
+                    *c = ACC ? *c + acc[i][j][e] : acc[i][j][e];
+                }
+            }
+    }
+}
+
+// ---- host -------------------------------------------------------------------------------
+size_t table_bytes(int64_t num_groups) {
+    return sizeof(TileTable) + static_cast<size_t>(num_groups + 1) * sizeof(GroupEntry);
+}
+
+template <int DT, int OUT>
+int launch16(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red, unsigned grid) {
+    const void *fn;
+    if (a_red && b_red) fn = reinterpret_cast<const void *>(&gmm16_kernel<DT, true, true, OUT>);
+    else if (a_red) fn = reinterpret_cast<const void *>(&gmm16_kernel<DT, true, false, OUT>);
+    else if (b_red) fn = reinterpret_cast<const void *>(&gmm16_kernel<DT, false, true, OUT>);
+    else fn = reinterpret_cast<const void *>(&gmm16_kernel<DT, false, false, OUT>);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes16);
+    MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "ms_gmm: hipFuncSetAttribute: %s", hipGetErrorString(e));
+    GmmArgs copy = args;
+    void *kargs[] = {&copy};
+    e = hipLaunchKernel(fn, dim3(grid), dim3(256), kargs, kLdsBytes16, stream);
+    MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "ms_gmm: launch failed: %s", hipGetErrorString(e));
+    return MS_OK;
+}
+
+}  // namespace
+}  // namespace ms
+
+using namespace ms;
+
+extern "C" int ms_gmm_workspace_size(int64_t num_groups, int64_t m, int group_type, size_t *bytes) {
+    (void)m;
+    (void)group_type;
+    MS_REQUIRE(bytes != nullptr, MS_ERR_INVALID_ARGUMENT, "ms_gmm_workspace_size: bytes is NULL");
+    MS_REQUIRE(num_groups >= 1 && num_groups <= kMaxGroups, MS_ERR_UNSUPPORTED,
+               "ms_gmm_workspace_size: num_groups %lld outside [1, %d]", (long long)num_groups, kMaxGroups);
+    *bytes = (table_bytes(num_groups) + 255) & ~static_cast<size_t>(255);
+    return MS_OK;
+}
+
+extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int64_t x_stride1, const void *weight,
+                      int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1, void *y, int64_t y_stride_row,
+                      const int64_t *group_list, int group_list_type, int group_type, int64_t num_groups, int64_t m,
+                      int64_t k, int64_t n, int dtype, int out_dtype, int accumulate, void *workspace,
+                      size_t workspace_bytes) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED, "ms_gmm: bad dtype %d", dtype);
+    MS_REQUIRE(out_dtype == dtype || out_dtype == MS_FP32, MS_ERR_UNSUPPORTED,
+               "ms_gmm: out_dtype must equal dtype or be fp32");
+    MS_REQUIRE(!accumulate || out_dtype == MS_FP32, MS_ERR_UNSUPPORTED, "ms_gmm: accumulate needs an fp32 output");
+    MS_REQUIRE(group_type == 0 || group_type == 2, MS_ERR_UNSUPPORTED, "ms_gmm: group_type must be 0 or 2, got %d", group_type);
+    MS_REQUIRE(group_list_type == 0 || group_list_type == 1, MS_ERR_INVALID_ARGUMENT,
+               "ms_gmm: group_list_type must be 0 or 1, got %d", group_list_type);
+    MS_REQUIRE(num_groups >= 1 && num_groups <= kMaxGroups, MS_ERR_UNSUPPORTED,
+               "ms_gmm: num_groups %lld outside [1, %d]", (long long)num_groups, kMaxGroups);
+    MS_REQUIRE(m >= 0 && k >= 0 && n >= 0 && m < (1ll << 31) - 512 && k < (1ll << 31) - 512 && n < (1ll << 31) - 512,
+               MS_ERR_INVALID_ARGUMENT, "ms_gmm: bad sizes m=%lld k=%lld n=%lld", (long long)m, (long long)k, (long long)n);
+    MS_REQUIRE(group_list != nullptr, MS_ERR_INVALID_ARGUMENT, "ms_gmm: group_list is NULL");
+    const size_t need = table_bytes(num_groups);
+    MS_REQUIRE(workspace != nullptr && workspace_bytes >= need, MS_ERR_WORKSPACE_TOO_SMALL,
+               "ms_gmm: workspace %zu < %zu bytes", workspace_bytes, need);
+    MS_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7u) == 0, MS_ERR_INVALID_ARGUMENT, "ms_gmm: workspace must be 8-byte aligned");
+
+    // Output extent; nothing to do for an empty output.
+    const int64_t out_rows = group_type == 0 ? m : k;       // rows per output block
+    const int64_t red_total = group_type == 0 ? k : m;
+    if (n == 0 || out_rows == 0) return MS_OK;
+    MS_REQUIRE(y != nullptr, MS_ERR_INVALID_ARGUMENT, "ms_gmm: y is NULL");
+    MS_REQUIRE(red_total == 0 || (x != nullptr && weight != nullptr), MS_ERR_INVALID_ARGUMENT, "ms_gmm: NULL operand");
+    MS_REQUIRE(y_stride_row >= n, MS_ERR_INVALID_ARGUMENT, "ms_gmm: y_stride_row %lld < n %lld", (long long)y_stride_row, (long long)n);
+
+    // x is [rows, red] for both group types ([m,k] / [k,m]); weight is [red, cols].
+    const int64_t a_stride_row = x_stride0, a_stride_red = x_stride1;
+    const int64_t b_stride_red = w_stride0, b_stride_col = w_stride1;
+    const bool a_red = a_stride_red == 1 || red_total <= 1;
+    const bool a_row = a_stride_row == 1 || out_rows <= 1;
+    const bool b_red = b_stride_red == 1 || red_total <= 1;
+    const bool b_col = b_stride_col == 1 || n <= 1;
+    MS_REQUIRE(a_red || a_row, MS_ERR_UNSUPPORTED, "ms_gmm: x needs one unit stride (got %lld, %lld)", (long long)x_stride0, (long long)x_stride1);
+    MS_REQUIRE(b_red || b_col, MS_ERR_UNSUPPORTED, "ms_gmm: weight needs one unit stride (got %lld, %lld)", (long long)w_stride0, (long long)w_stride1);
+
+    const bool is32 = dtype == MS_FP32;
+    const int tile_rows = is32 ? FM : BM;
+    const int tile_cols = is32 ? FN : BN;
+    const int64_t num_col_tiles = ceil_div(n, tile_cols);
+    const int64_t row_tiles_bound = group_type == 0 ? ceil_div(m, tile_rows) + num_groups + 1
+                                                    : num_groups * ceil_div(k, tile_rows);
+    const int64_t tiles_bound = row_tiles_bound * num_col_tiles;
+    MS_REQUIRE(tiles_bound < (1ll << 30), MS_ERR_UNSUPPORTED, "ms_gmm: problem too large (%lld tiles)", (long long)tiles_bound);
+
+    TileTable *table = static_cast<TileTable *>(workspace);
+    const int64_t c_stride_group = k * y_stride_row;
+    hipLaunchKernelGGL(gmm_schedule_kernel, dim3(1), dim3(256), static_cast<size_t>(num_groups) * sizeof(int64_t), stream,
+                       group_list, group_list_type, group_type, static_cast<int>(num_groups), static_cast<int>(m),
+                       static_cast<int>(k), tile_rows, static_cast<int>(num_col_tiles), w_stride_group, c_stride_group,
+                       table);
+    MS_CHECK_LAUNCH("gmm_schedule_kernel");
+
+    GmmArgs args{};
+    args.a = x;
+    args.b = weight;
+    args.c = y;
+    args.table = table;
+    args.a_stride_row = a_stride_row;
+    args.a_stride_red = a_stride_red;
+    args.b_stride_red = b_stride_red;
+    args.b_stride_col = b_stride_col;
+    args.c_stride_row = y_stride_row;
+    args.cols = static_cast<int>(n);
+    args.num_col_tiles = static_cast<int>(num_col_tiles);
+    const unsigned grid = static_cast<unsigned>(ceil_div(tiles_bound, 8) * 8);
+
+    if (is32) {
+        if (accumulate)
+            hipLaunchKernelGGL(gmm32_kernel<true>, dim3(grid), dim3(256), 0, stream, args);
+        else
+            hipLaunchKernelGGL(gmm32_kernel<false>, dim3(grid), dim3(256), 0, stream, args);
+        MS_CHECK_LAUNCH("gmm32_kernel");
+        return MS_OK;
+    }
+
+    // 16-byte vector eligibility of each operand.
+    const bool use_a_red = a_stride_red == 1;  // prefer the reduction-contiguous reading when both hold
+    const bool use_b_red = b_stride_red == 1;
+    const int64_t a_other = use_a_red ? a_stride_row : a_stride_red;
+    const int64_t b_other = use_b_red ? b_stride_col : b_stride_red;
+    args.a_vec_ok = aligned16(x) && a_other % 8 == 0;
+    args.b_vec_ok = aligned16(weight) && b_other % 8 == 0 && w_stride_group % 8 == 0;
+    const int out_size = out_dtype == MS_FP32 ? 4 : 2;
+    args.c_vec_ok = (reinterpret_cast<uintptr_t>(y) % (4 * out_size) == 0) && y_stride_row % 4 == 0 &&
+                    (group_type == 0 || c_stride_group % 4 == 0);
+    // A stride of 1 in a dim of extent 1 may come with an arbitrary other stride.
+    const bool a_is_red = use_a_red || !a_row;
+    const bool b_is_red = use_b_red || !b_col;
+    if (!use_a_red && a_stride_row != 1) args.a_vec_ok = 0;
+    if (!use_b_red && b_stride_col != 1) args.b_vec_ok = 0;
+
+    const int out = accumulate ? ACC_F32 : (out_dtype == MS_FP32 ? OUT_F32 : OUT_SAME);
+    if (dtype == MS_BF16) {
+        if (out == OUT_SAME) return launch16<MS_BF16, OUT_SAME>(stream, args, a_is_red, b_is_red, grid);
+        if (out == OUT_F32) return launch16<MS_BF16, OUT_F32>(stream, args, a_is_red, b_is_red, grid);
+        return launch16<MS_BF16, ACC_F32>(stream, args, a_is_red, b_is_red, grid);
+    }
+    if (out == OUT_SAME) return launch16<MS_FP16, OUT_SAME>(stream, args, a_is_red, b_is_red, grid);
+    if (out == OUT_F32) return launch16<MS_FP16, OUT_F32>(stream, args, a_is_red, b_is_red, grid);
+    return launch16<MS_FP16, ACC_F32>(stream, args, a_is_red, b_is_red, grid);
+}

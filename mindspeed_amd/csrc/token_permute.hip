@@ -1,0 +1,611 @@
+// MoE token permute / unpermute for gfx950 (MI355X).
+//
+// permute  = stable counting sort of the flattened expert ids (wavefront-ballot
+//            match, per-wave histogram rows, LDS prefix scan, no atomics, so
+//            the order is deterministic) followed by a coalesced 16-byte row
+//            scatter that reads every token row once and writes its topk
+//            copies.
+// unpermute = per-token top-k gather with fp32 accumulation in registers and
+//            one rounding; its backward scatters prob-scaled rows and reduces
+//            the per-(token, slot) dot products for grad_probs.
+//
+// All kernels are HBM-bound; rows move as 16-byte vectors per lane.
+#include "common.h"
+
+namespace ms {
+namespace {
+
+constexpr int kSortBlockWaves = 16;          // single-block sort: 1024 threads
+constexpr int kSmallSortMax = 16384;         // flat positions handled by one block
+constexpr int kHistWavesPerBlock = 4;        // multi-block sort: 256 threads
+constexpr int kMaxSegments = 4096;
+
+// ---- wavefront helpers ---------------------------------------------------------
+template <typename IdxT>
+__device__ __forceinline__ int load_key(const IdxT *idx, int64_t i, int nbins) {
+    long long v = static_cast<long long>(idx[i]);
+    v = v < 0 ? 0 : v;
+    v = v >= nbins ? nbins - 1 : v;
+    return static_cast<int>(v);
+}
+
+// Mask of the valid lanes of this wavefront that hold the same key as the caller.
+__device__ __forceinline__ unsigned long long match_key(int key, bool valid, int nbits) {
+    unsigned long long m = __ballot(valid);
+    for (int b = 0; b < nbits; ++b) {
+        const bool bit = (key >> b) & 1;
+        const unsigned long long bal = __ballot(valid && bit);
+        m &= bit ? bal : ~bal;
+    }
+    return m;
+}
+
+// Histogram of idx[begin, end) into one table row owned by this wavefront.
+template <typename IdxT>
+__device__ __forceinline__ void wave_histogram(volatile int *row, const IdxT *idx, int begin, int end,
+                                               int nbins, int nbits) {
+    const int lane = threadIdx.x & 63;
+    for (int base = begin; base < end; base += 64) {
+        const int i = base + lane;
+        const bool valid = i < end;
+        const int key = valid ? load_key(idx, i, nbins) : 0;
+        const unsigned long long m = match_key(key, valid, nbits);
+        if (valid && lane == __ffsll(static_cast<long long>(m)) - 1) row[key] += __popcll(m);
+    }
+}
+
+// Stable scatter of idx[begin, end): row[key] holds the next output row of `key`
+// for this wavefront's segment.
+template <typename IdxT>
+__device__ __forceinline__ void wave_scatter(volatile int *row, const IdxT *idx, int begin, int end,
+                                             int nbins, int nbits, int num_out, int32_t *row_id_map,
+                                             int32_t *sorted_indices) {
+    const int lane = threadIdx.x & 63;
+    const unsigned long long lt = (1ull << lane) - 1ull;
+    for (int base = begin; base < end; base += 64) {
+        const int i = base + lane;
+        const bool valid = i < end;
+        const int key = valid ? load_key(idx, i, nbins) : 0;
+        const unsigned long long m = match_key(key, valid, nbits);
+        const int first = valid ? row[key] : 0;
+        const int rank = first + __popcll(m & lt);
+        __builtin_amdgcn_wave_barrier();
+        if (valid && lane == __ffsll(static_cast<long long>(m)) - 1) row[key] = first + __popcll(m);
+        __builtin_amdgcn_wave_barrier();
+        if (valid) {
+            row_id_map[i] = rank;
+            if (sorted_indices != nullptr && rank < num_out) sorted_indices[rank] = i;
+        }
+    }
+}
+
+// Exclusive scan of one int per thread over a block of up to 1024 threads.
+__device__ __forceinline__ int block_exclusive_scan(int v, int *scratch /* >= 16 ints */) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    int incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+    }
+    if (lane == 63) scratch[wave] = incl;
+    __syncthreads();
+    if (wave == 0) {
+        const int nw = (blockDim.x + 63) >> 6;
+        int w = lane < nw ? scratch[lane] : 0;
+        int wi = w;
+#pragma unroll
+        for (int d = 1; d < 16; d <<= 1) {
+            const int up = __shfl_up(wi, d, 64);
+            if (lane >= d) wi += up;
+        }
+        if (lane < nw) scratch[lane] = wi - w;
+    }
+    __syncthreads();
+    return incl - v + scratch[wave];
+}
+
+// ---- single-block sort (small inputs): one launch ---------------------------------
+template <typename IdxT>
+__global__ __launch_bounds__(kSortBlockWaves * 64) void sort_small_kernel(
+    const IdxT *__restrict__ idx, int n, int nbins, int nbits, int num_out, int32_t *row_id_map,
+    int32_t *sorted_indices, int64_t *tokens_per_expert, int tpe_n) {
+    extern __shared__ int lds[];  // [kSortBlockWaves][nbins] table, then 16 ints of scan scratch
+    int *scratch = lds + kSortBlockWaves * nbins;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    for (int i = tid; i < kSortBlockWaves * nbins; i += blockDim.x) lds[i] = 0;
+    __syncthreads();
+    int seg = (n + kSortBlockWaves - 1) / kSortBlockWaves;
+    seg = (seg + 63) & ~63;
+    const int begin = min(wave * seg, n);
+    const int end = min(begin + seg, n);
+    wave_histogram(lds + wave * nbins, idx, begin, end, nbins, nbits);
+    __syncthreads();
+    int total = 0;
+    if (tid < nbins) {
+        for (int w = 0; w < kSortBlockWaves; ++w) {
+            const int c = lds[w * nbins + tid];
+            lds[w * nbins + tid] = total;
+            total += c;
+        }
+    }
+    const int excl = block_exclusive_scan(total, scratch);
+    if (tid < nbins) {
+        for (int w = 0; w < kSortBlockWaves; ++w) lds[w * nbins + tid] += excl;
+        if (tokens_per_expert != nullptr && tid < tpe_n) tokens_per_expert[tid] = total;
+    }
+    __syncthreads();
+    wave_scatter(lds + wave * nbins, idx, begin, end, nbins, nbits, num_out, row_id_map, sorted_indices);
+}
+
+// ---- multi-block sort (large inputs): histogram, scan, scatter ----------------------
+template <typename IdxT>
+__global__ __launch_bounds__(kHistWavesPerBlock * 64) void sort_hist_kernel(
+    const IdxT *__restrict__ idx, int n, int seg, int nseg, int nbins, int nbits, int *table) {
+    extern __shared__ int lds[];  // [kHistWavesPerBlock][nbins]
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int s = blockIdx.x * kHistWavesPerBlock + wave;
+    int *row = lds + wave * nbins;
+    for (int e = lane; e < nbins; e += 64) row[e] = 0;
+    __builtin_amdgcn_wave_barrier();
+    if (s < nseg) {
+        const int begin = min(s * seg, n);
+        const int end = min(begin + seg, n);
+        wave_histogram(row, idx, begin, end, nbins, nbits);
+        __builtin_amdgcn_wave_barrier();
+        for (int e = lane; e < nbins; e += 64) table[static_cast<int64_t>(s) * nbins + e] = row[e];
+    }
+}
+
+__global__ __launch_bounds__(1024) void sort_scan_kernel(int *table, int nseg, int nbins,
+                                                         int64_t *tokens_per_expert, int tpe_n) {
+    __shared__ int scratch[16];
+    const int tid = threadIdx.x;
+    int total = 0;
+    if (tid < nbins) {
+        for (int s = 0; s < nseg; ++s) {
+            const int64_t at = static_cast<int64_t>(s) * nbins + tid;
+            const int c = table[at];
+            table[at] = total;
+            total += c;
+        }
+    }
+    const int excl = block_exclusive_scan(total, scratch);
+    if (tid < nbins) {
+        for (int s = 0; s < nseg; ++s) table[static_cast<int64_t>(s) * nbins + tid] += excl;
+        if (tokens_per_expert != nullptr && tid < tpe_n) tokens_per_expert[tid] = total;
+    }
+}
+
+template <typename IdxT>
+__global__ __launch_bounds__(kHistWavesPerBlock * 64) void sort_scatter_kernel(
+    const IdxT *__restrict__ idx, int n, int seg, int nseg, int nbins, int nbits, const int *table,
+    int num_out, int32_t *row_id_map, int32_t *sorted_indices) {
+    extern __shared__ int lds[];
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int s = blockIdx.x * kHistWavesPerBlock + wave;
+    if (s >= nseg) return;
+    int *row = lds + wave * nbins;
+    for (int e = lane; e < nbins; e += 64) row[e] = table[static_cast<int64_t>(s) * nbins + e];
+    __builtin_amdgcn_wave_barrier();
+    const int begin = min(s * seg, n);
+    const int end = min(begin + seg, n);
+    wave_scatter(row, idx, begin, end, nbins, nbits, num_out, row_id_map, sorted_indices);
+}
+
+// ---- row movers ---------------------------------------------------------------------
+// Thread layout shared by the row kernels: a block of 256 threads covers
+// rows_per_block rows, `lanes` threads per row, each thread striding over the
+// row's vectors.
+struct RowLayout {
+    int lanes;           // threads per row (power of two, 1..256)
+    int rows_per_block;  // 256 / lanes
+};
+inline RowLayout row_layout(int64_t vecs_per_row) {
+    int lanes = 1;
+    while (lanes < 256 && lanes < vecs_per_row) lanes <<= 1;
+    return RowLayout{lanes, 256 / lanes};
+}
+
+// permuted[row_id_map[t*k+j]] = tokens[t] for every kept (t, j).
+template <typename VecT>
+__global__ __launch_bounds__(256) void permute_rows_kernel(const VecT *__restrict__ tokens,
+                                                           VecT *__restrict__ permuted,
+                                                           const int32_t *__restrict__ row_id_map,
+                                                           int num_tokens, int topk, int vecs_per_row,
+                                                           int num_out, int lanes) {
+    const int local_row = threadIdx.x / lanes;
+    const int lane = threadIdx.x % lanes;
+    const int t = blockIdx.x * (256 / lanes) + local_row;
+    if (t >= num_tokens) return;
+    const VecT *src = tokens + static_cast<int64_t>(t) * vecs_per_row;
+    for (int c = lane; c < vecs_per_row; c += lanes) {
+        const VecT v = __builtin_nontemporal_load(src + c);
+        for (int j = 0; j < topk; ++j) {
+            const int d = row_id_map[static_cast<int64_t>(t) * topk + j];
+            if (d < num_out) __builtin_nontemporal_store(v, permuted + static_cast<int64_t>(d) * vecs_per_row + c);
+        }
+    }
+}
+
+// out[t] = sum_j w[t,j] * rows[row_id_map[t*k+j]] ; w == nullptr -> unweighted.
+// VEC: elements per thread access (16 bytes worth, or 1 for the unaligned path).
+template <typename DT, int VEC>
+__global__ __launch_bounds__(256) void gather_combine_kernel(
+    const typename DT::storage *__restrict__ rows, const int32_t *__restrict__ row_id_map,
+    const typename DT::storage *__restrict__ probs, typename DT::storage *__restrict__ out,
+    int num_tokens, int topk, int hidden, int num_rows, int lanes) {
+    using S = typename DT::storage;
+    const int local_row = threadIdx.x / lanes;
+    const int lane = threadIdx.x % lanes;
+    const int t = blockIdx.x * (256 / lanes) + local_row;
+    if (t >= num_tokens) return;
+    const int vecs = hidden / VEC;
+    for (int c = lane; c < vecs; c += lanes) {
+        float acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+        for (int j = 0; j < topk; ++j) {
+            const int d = row_id_map[static_cast<int64_t>(t) * topk + j];
+            if (d >= num_rows) continue;
+            const float w = probs != nullptr ? DT::to_float(probs[static_cast<int64_t>(t) * topk + j]) : 1.f;
+            const S *src = rows + static_cast<int64_t>(d) * hidden + static_cast<int64_t>(c) * VEC;
+            S tmp[VEC];
+            if constexpr (VEC * sizeof(S) == 16) {
+                *reinterpret_cast<v16 *>(tmp) = __builtin_nontemporal_load(reinterpret_cast<const v16 *>(src));
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) tmp[e] = src[e];
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] = fmaf(w, DT::to_float(tmp[e]), acc[e]);
+        }
+        S res[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) res[e] = DT::from_float(acc[e]);
+        S *dst = out + static_cast<int64_t>(t) * hidden + static_cast<int64_t>(c) * VEC;
+        if constexpr (VEC * sizeof(S) == 16) {
+            __builtin_nontemporal_store(*reinterpret_cast<v16 *>(res), reinterpret_cast<v16 *>(dst));
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) dst[e] = res[e];
+        }
+    }
+}
+
+// One block per token: grad_permuted[row] = w * dY[t]; grad_probs[t,j] = <dY[t], permuted[row]>.
+template <typename DT, int VEC>
+__global__ __launch_bounds__(256) void unpermute_grad_kernel(
+    const typename DT::storage *__restrict__ permuted, const typename DT::storage *__restrict__ grad_out,
+    const int32_t *__restrict__ row_id_map, const typename DT::storage *__restrict__ probs,
+    typename DT::storage *__restrict__ grad_permuted, typename DT::storage *__restrict__ grad_probs,
+    int topk, int hidden, int num_rows) {
+    using S = typename DT::storage;
+    __shared__ float partial[4];
+    const int t = blockIdx.x;
+    const int vecs = hidden / VEC;
+    const S *gy = grad_out + static_cast<int64_t>(t) * hidden;
+    for (int j = 0; j < topk; ++j) {
+        const int64_t flat = static_cast<int64_t>(t) * topk + j;
+        const int d = row_id_map[flat];
+        const bool kept = d < num_rows;
+        const float w = probs != nullptr ? DT::to_float(probs[flat]) : 1.f;
+        float dot = 0.f;
+        if (kept) {
+            for (int c = threadIdx.x; c < vecs; c += blockDim.x) {
+                S g[VEC], x[VEC], o[VEC];
+                const S *gp = gy + static_cast<int64_t>(c) * VEC;
+                const int64_t off = static_cast<int64_t>(d) * hidden + static_cast<int64_t>(c) * VEC;
+                if constexpr (VEC * sizeof(S) == 16) {
+                    *reinterpret_cast<v16 *>(g) = *reinterpret_cast<const v16 *>(gp);
+                    if (grad_probs != nullptr)
+                        *reinterpret_cast<v16 *>(x) =
+                            __builtin_nontemporal_load(reinterpret_cast<const v16 *>(permuted + off));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) g[e] = gp[e];
+                    if (grad_probs != nullptr) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) x[e] = permuted[off + e];
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float gf = DT::to_float(g[e]);
+                    o[e] = DT::from_float(w * gf);
+                    if (grad_probs != nullptr) dot = fmaf(gf, DT::to_float(x[e]), dot);
+                }
+                if constexpr (VEC * sizeof(S) == 16) {
+                    __builtin_nontemporal_store(*reinterpret_cast<v16 *>(o),
+                                                reinterpret_cast<v16 *>(grad_permuted + off));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) grad_permuted[off + e] = o[e];
+                }
+            }
+        }
+        if (grad_probs != nullptr) {
+#pragma unroll
+            for (int dlt = 32; dlt > 0; dlt >>= 1) dot += __shfl_down(dot, dlt, 64);
+            const int wave = threadIdx.x >> 6;
+            if ((threadIdx.x & 63) == 0) partial[wave] = dot;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                float s = 0.f;
+                for (int w2 = 0; w2 < (blockDim.x + 63) / 64; ++w2) s += partial[w2];
+                grad_probs[flat] = DT::from_float(s);
+            }
+            __syncthreads();
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void copy_bytes_kernel(const v16 *__restrict__ src, v16 *__restrict__ dst,
+                                                         size_t nvec) {
+    for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < nvec;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x)
+        dst[i] = src[i];
+}
+__global__ void copy_tail_kernel(const unsigned char *src, unsigned char *dst, size_t begin, size_t end) {
+    const size_t i = begin + blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
+    if (i < end) dst[i] = src[i];
+}
+
+// ---- host helpers -------------------------------------------------------------------
+struct SortPlan {
+    int n, nbins, nbits, seg, nseg;
+    bool small;
+};
+
+inline SortPlan make_sort_plan(int64_t n, int64_t experts_hint) {
+    SortPlan p{};
+    p.n = static_cast<int>(n);
+    int64_t want = experts_hint > 0 ? experts_hint : MS_MAX_EXPERTS;
+    p.nbins = 2;
+    p.nbits = 1;
+    while (p.nbins < want) {
+        p.nbins <<= 1;
+        p.nbits++;
+    }
+    p.small = n <= kSmallSortMax;
+    int64_t seg = 1024;
+    if (ceil_div(n, seg) > kMaxSegments) seg = (ceil_div(n, kMaxSegments) + 63) / 64 * 64;
+    p.seg = static_cast<int>(seg);
+    p.nseg = static_cast<int>(ceil_div(n, seg));
+    return p;
+}
+
+template <typename IdxT>
+int launch_sort(hipStream_t stream, const SortPlan &p, const IdxT *idx, int num_out, int32_t *row_id_map,
+                int32_t *sorted_indices, int64_t *tpe, int tpe_n, void *workspace) {
+    if (p.n == 0) return MS_OK;
+    if (p.small) {
+        const size_t lds = (static_cast<size_t>(kSortBlockWaves) * p.nbins + 16) * sizeof(int);
+        static thread_local bool configured[2] = {false, false};
+        constexpr int which = sizeof(IdxT) == 8 ? 1 : 0;
+        if (!configured[which]) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&sort_small_kernel<IdxT>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               (kSortBlockWaves * MS_MAX_EXPERTS + 16) * sizeof(int));
+            MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "hipFuncSetAttribute(sort_small): %s", hipGetErrorString(e));
+            configured[which] = true;
+        }
+        hipLaunchKernelGGL(sort_small_kernel<IdxT>, dim3(1), dim3(kSortBlockWaves * 64), lds, stream, idx, p.n,
+                           p.nbins, p.nbits, num_out, row_id_map, sorted_indices, tpe, tpe_n);
+        MS_CHECK_LAUNCH("sort_small_kernel");
+        return MS_OK;
+    }
+    int *table = static_cast<int *>(workspace);
+    const int blocks = static_cast<int>(ceil_div(p.nseg, kHistWavesPerBlock));
+    const size_t lds = static_cast<size_t>(kHistWavesPerBlock) * p.nbins * sizeof(int);
+    hipLaunchKernelGGL(sort_hist_kernel<IdxT>, dim3(blocks), dim3(kHistWavesPerBlock * 64), lds, stream, idx, p.n,
+                       p.seg, p.nseg, p.nbins, p.nbits, table);
+    MS_CHECK_LAUNCH("sort_hist_kernel");
+    hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(1024), 0, stream, table, p.nseg, p.nbins, tpe, tpe_n);
+    MS_CHECK_LAUNCH("sort_scan_kernel");
+    hipLaunchKernelGGL(sort_scatter_kernel<IdxT>, dim3(blocks), dim3(kHistWavesPerBlock * 64), lds, stream, idx,
+                       p.n, p.seg, p.nseg, p.nbins, p.nbits, table, num_out, row_id_map, sorted_indices);
+    MS_CHECK_LAUNCH("sort_scatter_kernel");
+    return MS_OK;
+}
+
+template <typename VecT>
+int launch_permute_rows(hipStream_t stream, const void *tokens, void *permuted, const int32_t *map, int64_t T,
+                        int64_t k, int64_t row_bytes, int64_t num_out) {
+    const int64_t vecs = row_bytes / sizeof(VecT);
+    const RowLayout rl = row_layout(vecs);
+    const int64_t blocks = ceil_div(T, rl.rows_per_block);
+    hipLaunchKernelGGL(permute_rows_kernel<VecT>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
+                       static_cast<const VecT *>(tokens), static_cast<VecT *>(permuted), map, static_cast<int>(T),
+                       static_cast<int>(k), static_cast<int>(vecs), static_cast<int>(num_out), rl.lanes);
+    MS_CHECK_LAUNCH("permute_rows_kernel");
+    return MS_OK;
+}
+
+template <typename DT>
+int launch_gather_combine(hipStream_t stream, const void *rows, const int32_t *map, const void *probs, void *out,
+                          int64_t T, int64_t k, int64_t H, int64_t num_rows) {
+    using S = typename DT::storage;
+    constexpr int VEC = 16 / sizeof(S);
+    const bool vec_ok = (H % VEC == 0) && aligned16(rows) && aligned16(out);
+    const int64_t vecs = vec_ok ? H / VEC : H;
+    const RowLayout rl = row_layout(vecs);
+    const unsigned blocks = static_cast<unsigned>(ceil_div(T, rl.rows_per_block));
+    if (vec_ok) {
+        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC>), dim3(blocks), dim3(256), 0, stream,
+                           static_cast<const S *>(rows), map, static_cast<const S *>(probs), static_cast<S *>(out),
+                           static_cast<int>(T), static_cast<int>(k), static_cast<int>(H),
+                           static_cast<int>(num_rows), rl.lanes);
+    } else {
+        hipLaunchKernelGGL((gather_combine_kernel<DT, 1>), dim3(blocks), dim3(256), 0, stream,
+                           static_cast<const S *>(rows), map, static_cast<const S *>(probs), static_cast<S *>(out),
+                           static_cast<int>(T), static_cast<int>(k), static_cast<int>(H),
+                           static_cast<int>(num_rows), rl.lanes);
+    }
+    MS_CHECK_LAUNCH("gather_combine_kernel");
+    return MS_OK;
+}
+
+template <typename DT>
+int launch_unpermute_grad(hipStream_t stream, const void *permuted, const void *gy, const int32_t *map,
+                          const void *probs, void *gperm, void *gprobs, int64_t T, int64_t k, int64_t H,
+                          int64_t num_rows) {
+    using S = typename DT::storage;
+    constexpr int VEC = 16 / sizeof(S);
+    const bool vec_ok = (H % VEC == 0) && aligned16(gy) && aligned16(gperm) && (permuted == nullptr || aligned16(permuted));
+    const int64_t vecs = vec_ok ? H / VEC : H;
+    int threads = 64;
+    while (threads < 256 && threads < vecs) threads <<= 1;
+    if (vec_ok) {
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC>), dim3(static_cast<unsigned>(T)), dim3(threads), 0, stream,
+                           static_cast<const S *>(permuted), static_cast<const S *>(gy), map,
+                           static_cast<const S *>(probs), static_cast<S *>(gperm), static_cast<S *>(gprobs),
+                           static_cast<int>(k), static_cast<int>(H), static_cast<int>(num_rows));
+    } else {
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, 1>), dim3(static_cast<unsigned>(T)), dim3(threads), 0, stream,
+                           static_cast<const S *>(permuted), static_cast<const S *>(gy), map,
+                           static_cast<const S *>(probs), static_cast<S *>(gperm), static_cast<S *>(gprobs),
+                           static_cast<int>(k), static_cast<int>(H), static_cast<int>(num_rows));
+    }
+    MS_CHECK_LAUNCH("unpermute_grad_kernel");
+    return MS_OK;
+}
+
+int check_common(const char *fn, int64_t T, int64_t k, int64_t H, int dtype) {
+    MS_REQUIRE(T >= 0 && k >= 1 && H >= 1, MS_ERR_INVALID_ARGUMENT,
+               "%s: need num_tokens >= 0, topk >= 1, hidden >= 1 (got %lld, %lld, %lld)", fn, (long long)T,
+               (long long)k, (long long)H);
+    MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED,
+               "%s: dtype %d is not one of bf16/fp16/fp32", fn, dtype);
+    MS_REQUIRE(T * k < (1ll << 31) - 64 && H < (1ll << 31), MS_ERR_UNSUPPORTED,
+               "%s: num_tokens*topk and hidden must fit int32", fn);
+    return MS_OK;
+}
+
+}  // namespace
+}  // namespace ms
+
+using namespace ms;
+
+extern "C" int ms_moe_token_permute_workspace_size(int64_t num_tokens, int64_t topk, int64_t num_experts_hint,
+                                                   size_t *bytes) {
+    MS_REQUIRE(bytes != nullptr, MS_ERR_INVALID_ARGUMENT, "ms_moe_token_permute_workspace_size: bytes is NULL");
+    MS_REQUIRE(num_tokens >= 0 && topk >= 1, MS_ERR_INVALID_ARGUMENT,
+               "ms_moe_token_permute_workspace_size: bad sizes");
+    MS_REQUIRE(num_experts_hint >= 0 && num_experts_hint <= MS_MAX_EXPERTS, MS_ERR_UNSUPPORTED,
+               "ms_moe_token_permute_workspace_size: num_experts_hint %lld exceeds %d", (long long)num_experts_hint,
+               MS_MAX_EXPERTS);
+    const SortPlan p = make_sort_plan(num_tokens * topk, num_experts_hint);
+    *bytes = p.small ? 0 : static_cast<size_t>(p.nseg) * p.nbins * sizeof(int);
+    return MS_OK;
+}
+
+extern "C" int ms_moe_token_permute(ms_stream_t stream_, const void *tokens, const void *indices, int index_dtype,
+                                    int64_t T, int64_t k, int64_t H, int dtype, int64_t num_out,
+                                    int64_t experts_hint, void *permuted, int32_t *row_id_map,
+                                    int32_t *sorted_indices, int64_t *tokens_per_expert, void *workspace,
+                                    size_t workspace_bytes) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (int rc = check_common("ms_moe_token_permute", T, k, H, dtype)) return rc;
+    MS_REQUIRE(index_dtype == MS_INT32 || index_dtype == MS_INT64, MS_ERR_UNSUPPORTED,
+               "ms_moe_token_permute: indices must be int32 or int64");
+    MS_REQUIRE(experts_hint >= 0 && experts_hint <= MS_MAX_EXPERTS, MS_ERR_UNSUPPORTED,
+               "ms_moe_token_permute: num_experts_hint %lld exceeds %d", (long long)experts_hint, MS_MAX_EXPERTS);
+    MS_REQUIRE(num_out >= 0 && num_out <= T * k, MS_ERR_INVALID_ARGUMENT,
+               "ms_moe_token_permute: num_out_tokens %lld outside [0, %lld]", (long long)num_out, (long long)(T * k));
+    MS_REQUIRE(tokens_per_expert == nullptr || experts_hint > 0, MS_ERR_INVALID_ARGUMENT,
+               "ms_moe_token_permute: tokens_per_expert needs num_experts_hint > 0");
+    if (T == 0) return MS_OK;
+    MS_REQUIRE(tokens && indices && row_id_map && (permuted || num_out == 0), MS_ERR_INVALID_ARGUMENT,
+               "ms_moe_token_permute: NULL tensor pointer");
+    const SortPlan p = make_sort_plan(T * k, experts_hint);
+    const size_t need = p.small ? 0 : static_cast<size_t>(p.nseg) * p.nbins * sizeof(int);
+    MS_REQUIRE(workspace_bytes >= need && (need == 0 || workspace != nullptr), MS_ERR_WORKSPACE_TOO_SMALL,
+               "ms_moe_token_permute: workspace %zu < %zu bytes", workspace_bytes, need);
+    int rc;
+    if (index_dtype == MS_INT32)
+        rc = launch_sort(stream, p, static_cast<const int32_t *>(indices), (int)num_out, row_id_map, sorted_indices,
+                         tokens_per_expert, (int)experts_hint, workspace);
+    else
+        rc = launch_sort(stream, p, static_cast<const int64_t *>(indices), (int)num_out, row_id_map, sorted_indices,
+                         tokens_per_expert, (int)experts_hint, workspace);
+    if (rc) return rc;
+    if (num_out == 0) return MS_OK;
+    const int64_t row_bytes = H * dtype_size(dtype);
+    if (row_bytes % 16 == 0 && aligned16(tokens) && aligned16(permuted))
+        return launch_permute_rows<v16>(stream, tokens, permuted, row_id_map, T, k, row_bytes, num_out);
+    if (dtype == MS_FP32) return launch_permute_rows<uint32_t>(stream, tokens, permuted, row_id_map, T, k, row_bytes, num_out);
+    return launch_permute_rows<uint16_t>(stream, tokens, permuted, row_id_map, T, k, row_bytes, num_out);
+}
+
+extern "C" int ms_moe_token_unpermute(ms_stream_t stream_, const void *permuted, const int32_t *row_id_map,
+                                      const void *probs, int64_t T, int64_t k, int64_t H, int dtype,
+                                      int64_t num_rows, void *out) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (int rc = check_common("ms_moe_token_unpermute", T, k, H, dtype)) return rc;
+    MS_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31), MS_ERR_INVALID_ARGUMENT, "ms_moe_token_unpermute: bad num_permuted_rows");
+    if (T == 0) return MS_OK;
+    MS_REQUIRE((permuted || num_rows == 0) && row_id_map && out, MS_ERR_INVALID_ARGUMENT,
+               "ms_moe_token_unpermute: NULL tensor pointer");
+    switch (dtype) {
+        case MS_BF16: return launch_gather_combine<BF16>(stream, permuted, row_id_map, probs, out, T, k, H, num_rows);
+        case MS_FP16: return launch_gather_combine<FP16>(stream, permuted, row_id_map, probs, out, T, k, H, num_rows);
+        default: return launch_gather_combine<FP32>(stream, permuted, row_id_map, probs, out, T, k, H, num_rows);
+    }
+}
+
+extern "C" int ms_moe_token_permute_grad(ms_stream_t stream, const void *grad_permuted, const int32_t *row_id_map,
+                                         int64_t T, int64_t k, int64_t H, int dtype, int64_t num_rows,
+                                         void *grad_tokens) {
+    // The backward of a row gather is the unweighted top-k gather-sum.
+    return ms_moe_token_unpermute(stream, grad_permuted, row_id_map, nullptr, T, k, H, dtype, num_rows, grad_tokens);
+}
+
+extern "C" int ms_moe_token_unpermute_grad(ms_stream_t stream_, const void *permuted, const void *grad_out,
+                                           const int32_t *row_id_map, const void *probs, int64_t T, int64_t k,
+                                           int64_t H, int dtype, int64_t num_rows, void *grad_permuted,
+                                           void *grad_probs) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (int rc = check_common("ms_moe_token_unpermute_grad", T, k, H, dtype)) return rc;
+    MS_REQUIRE(num_rows >= 0 && num_rows <= T * k, MS_ERR_INVALID_ARGUMENT,
+               "ms_moe_token_unpermute_grad: num_permuted_rows %lld outside [0, %lld]", (long long)num_rows,
+               (long long)(T * k));
+    MS_REQUIRE((grad_probs == nullptr) == (probs == nullptr), MS_ERR_INVALID_ARGUMENT,
+               "ms_moe_token_unpermute_grad: probs and grad_probs must be given together");
+    MS_REQUIRE(grad_probs == nullptr || permuted != nullptr || num_rows == 0, MS_ERR_INVALID_ARGUMENT,
+               "ms_moe_token_unpermute_grad: grad_probs needs permuted_tokens");
+    if (T == 0) return MS_OK;
+    MS_REQUIRE(grad_out && row_id_map && (grad_permuted || num_rows == 0), MS_ERR_INVALID_ARGUMENT,
+               "ms_moe_token_unpermute_grad: NULL tensor pointer");
+    switch (dtype) {
+        case MS_BF16: return launch_unpermute_grad<BF16>(stream, permuted, grad_out, row_id_map, probs, grad_permuted, grad_probs, T, k, H, num_rows);
+        case MS_FP16: return launch_unpermute_grad<FP16>(stream, permuted, grad_out, row_id_map, probs, grad_permuted, grad_probs, T, k, H, num_rows);
+        default: return launch_unpermute_grad<FP32>(stream, permuted, grad_out, row_id_map, probs, grad_permuted, grad_probs, T, k, H, num_rows);
+    }
+}
+
+extern "C" int ms_copy_bytes(ms_stream_t stream_, const void *src, void *dst, size_t bytes) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (bytes == 0) return MS_OK;
+    MS_REQUIRE(src && dst, MS_ERR_INVALID_ARGUMENT, "ms_copy_bytes: NULL pointer");
+    size_t nvec = (aligned16(src) && aligned16(dst)) ? bytes / 16 : 0;
+    if (nvec) {
+        size_t blocks = (nvec + 255) / 256;
+        if (blocks > 256 * 32) blocks = 256 * 32;
+        hipLaunchKernelGGL(copy_bytes_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
+                           static_cast<const v16 *>(src), static_cast<v16 *>(dst), nvec);
+        MS_CHECK_LAUNCH("copy_bytes_kernel");
+    }
+    const size_t done = nvec * 16;
+    if (done < bytes) {
+        const size_t rest = bytes - done;
+        hipLaunchKernelGGL(copy_tail_kernel, dim3(static_cast<unsigned>((rest + 255) / 256)), dim3(256), 0, stream,
+                           static_cast<const unsigned char *>(src), static_cast<unsigned char *>(dst), done, bytes);
+        MS_CHECK_LAUNCH("copy_tail_kernel");
+    }
+    return MS_OK;
+}

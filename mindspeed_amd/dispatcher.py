@@ -1,0 +1,31 @@
+"""Single-rank ``dispatch_mlp_combine``: permute -> grouped MLP -> weighted unpermute.
+
+Mirrors mindspeed/fsdp/distributed/expert_parallel/dispatcher.py:37-52,81-113 for
+one rank (``ep_size == 1``: no all-to-all, and the second permute / unpermute
+pair of the reference is the identity because rows are already expert-major).
+``tokens_per_expert`` comes out of the permute kernel's histogram instead of a
+separate ``torch.bincount`` (dispatcher.py:64), and stays on the device.
+"""
+from __future__ import annotations
+
+import torch
+
+from .ops import (fused_swiglu, moe_token_permute_with_aux, npu_gmm_v2, npu_moe_token_unpermute)
+
+__all__ = ["experts_computation", "dispatch_mlp_combine"]
+
+
+def experts_computation(hidden_states, split_list, gate_up_weights, down_weights):
+    """``gmm -> silu(gate) * up -> gmm`` (dispatcher.py:93-104); ``split_list`` = rows per expert."""
+    fc1 = npu_gmm_v2(hidden_states, gate_up_weights, group_list=split_list, group_type=0)
+    act = fused_swiglu(fc1)
+    return npu_gmm_v2(act, down_weights, group_list=split_list, group_type=0)
+
+
+def dispatch_mlp_combine(hidden_states, top_k_index, top_k_weights, weights, num_global_experts=None):
+    gate_up_weights, down_weights = weights
+    num_experts = gate_up_weights.size(0) if num_global_experts is None else num_global_experts
+    permuted, row_id_map, _, tokens_per_expert = moe_token_permute_with_aux(
+        hidden_states, top_k_index, num_experts=num_experts)
+    out = experts_computation(permuted, tokens_per_expert, gate_up_weights, down_weights)
+    return npu_moe_token_unpermute(out, row_id_map, top_k_weights)

@@ -1,0 +1,324 @@
+"""``npu_gmm`` / ``npu_gmm_v2`` on MI355X.
+
+Mirrors mindspeed/ops/gmm.py: the same parameter verification
+(``npu_gmm_param_verification``, gmm.py:103-136), the same dispatcher schemas
+(mindspeed/op_builder/gmm_builder.py:90-93,131-133), the same autograd split
+into forward / dX / dW (gmm.py:20-99, mindspeed/ops/csrc/cann/gmm.cpp:169-293)
+and the same raw list-in / list-out module that
+``GMMFunction.builder.load()`` returns (gmm.cpp:295-309).  Every product is one
+call of the ``ms_gmm`` C-ABI entry point on strided views; nothing is
+transposed in memory.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from .. import _lib, flop_counter
+from .npu_groupmatmul_add import npu_groupmatmul_add_fp32
+
+__all__ = ["npu_gmm", "npu_gmm_v2", "GMMFunction"]
+
+
+# --------------------------------------------------------------------------
+# raw kernel call
+# --------------------------------------------------------------------------
+def _unit_stride_view(t: torch.Tensor) -> torch.Tensor:
+    """Return ``t`` if one of its two matrix strides is 1, else a contiguous copy."""
+    if t.stride(-1) == 1 or t.stride(-2) == 1 or t.size(-1) <= 1 or t.size(-2) <= 1:
+        return t
+    return t.contiguous()
+
+
+def _group_list_tensor(group_list, device) -> torch.Tensor:
+    if isinstance(group_list, torch.Tensor):
+        if group_list.device != device:
+            group_list = group_list.to(device)
+        return group_list.contiguous()
+    return torch.tensor(list(group_list), dtype=torch.int64, device=device)
+
+
+def gmm_raw(x, weight, group_list, group_type, group_list_type, out=None, accumulate=False):
+    """One grouped matmul on the current stream.
+
+    group_type 0: ``x [M, K]``, ``weight [E, K, N]`` -> ``[M, N]``.
+    group_type 2: ``x [K, M]``, ``weight [M, N]`` -> ``[E, K, N]``.
+    ``out`` (fp32, contiguous) with ``accumulate`` adds the result in place.
+    """
+    lib = _lib.load()
+    _lib.require_device(x, "x")
+    _lib.require_device(weight, "weight")
+    dev = x.device
+    dtype = _lib.dtype_code(x.dtype, "x")
+    if weight.dtype != x.dtype:
+        raise TypeError(f"x and weight must have the same dtype, got {x.dtype} and {weight.dtype}")
+    gl = _group_list_tensor(group_list, dev)
+    if gl.dtype != torch.int64 or gl.dim() != 1:
+        raise TypeError("group_list must be a one-dimensional int64 tensor")
+    num_groups = gl.numel()
+    x = _unit_stride_view(x)
+    weight = _unit_stride_view(weight)
+    if group_type == 0:
+        if x.dim() != 2 or weight.dim() != 3:
+            raise ValueError(f"group_type 0 needs x [M, K] and weight [E, K, N], got {tuple(x.shape)}, {tuple(weight.shape)}")
+        m, k = x.shape
+        if weight.size(0) != num_groups or weight.size(1) != k:
+            raise ValueError(f"weight {tuple(weight.shape)} does not match x {tuple(x.shape)} and {num_groups} groups")
+        n = weight.size(2)
+        w_strides = (weight.stride(0), weight.stride(1), weight.stride(2))
+        out_shape = (m, n)
+    elif group_type == 2:
+        if x.dim() != 2 or weight.dim() != 2:
+            raise ValueError(f"group_type 2 needs x [K, M] and weight [M, N], got {tuple(x.shape)}, {tuple(weight.shape)}")
+        k, m = x.shape
+        if weight.size(0) != m:
+            raise ValueError(f"weight {tuple(weight.shape)} does not match x {tuple(x.shape)}")
+        n = weight.size(1)
+        w_strides = (0, weight.stride(0), weight.stride(1))
+        out_shape = (num_groups, k, n)
+    else:
+        raise ValueError(f"group_type must be 0 or 2, got {group_type}")
+    if out is None:
+        out = torch.empty(out_shape, dtype=x.dtype, device=dev)
+        out_dtype = dtype
+    else:
+        if out.dtype != torch.float32 or not out.is_contiguous() or out.numel() != out_shape[0] * out_shape[1] * (out_shape[2] if len(out_shape) == 3 else 1):
+            raise ValueError("out must be a contiguous fp32 tensor of the result's size")
+        out_dtype = _lib.MS_FP32
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(lib.ms_gmm_workspace_size(num_groups, m, group_type, ctypes.byref(nbytes)), "ms_gmm_workspace_size")
+    ws = _lib.workspace(nbytes.value, dev)
+    # kernel flavour by operand layout: NN (forward), NT (weight read transposed: dX), TN (dW)
+    if group_type == 2:
+        kind = "gmm_dw"
+    elif w_strides[1] == 1 and w_strides[2] != 1:
+        kind = "gmm_dx"
+    else:
+        kind = "gmm_fwd"
+    with torch.cuda.device(dev), flop_counter.op(kind, flop_counter.gmm_flops(m, k, n), "flop", dev):
+        _lib.check(lib.ms_gmm(
+            _lib.stream_ptr(dev), _lib.ptr(x), x.stride(0), x.stride(1), _lib.ptr(weight), *w_strides,
+            _lib.ptr(out), n, _lib.ptr(gl), group_list_type, group_type, num_groups, m, k, n, dtype, out_dtype,
+            1 if accumulate else 0, _lib.ptr(ws), ws.numel()), "ms_gmm")
+    return out
+
+
+class _RawGmmModule:
+    """Stand-in for the pybind module of mindspeed/ops/csrc/cann/gmm.cpp:295-309.
+
+    Callers such as mindspeed/core/transformer/moe/grouped_matmul_util.py:140-184
+    use ``GMMFunction.builder.load().npu_gmm([x], [w], bias, group_list, group_type,
+    group_list_type)`` and get lists back.
+    """
+
+    @staticmethod
+    def npu_gmm(x, weight, bias, group_list, group_type, group_list_type):
+        if bias:
+            raise ValueError("bias is not supported by the grouped matmul kernels")
+        if len(x) != 1 or len(weight) != 1:
+            raise RuntimeError("Neither x nor weight could be empty; single-tensor (split_item=3) form only.")
+        return [gmm_raw(x[0], weight[0], group_list, group_type if group_type is not None else 0,
+                        group_list_type or 0)]
+
+    @staticmethod
+    def npu_gmm_backward(grad, x, weight, group_list, group_list_type):
+        # gmm.cpp:169-246: dx = gmm(grad, w^T, 0); dw = gmm(x^T, grad, 2).reshape(w.shape)
+        glt = group_list_type or 0
+        dx = gmm_raw(grad[0], weight[0].transpose(-1, -2), group_list, 0, glt)
+        dw = gmm_raw(x[0].transpose(-1, -2), grad[0], group_list, 2, glt).reshape(weight[0].shape)
+        return [dx], [dw], []
+
+    @staticmethod
+    def npu_gmm_backward_fusion(grad, weight, group_list, group_list_type):
+        # gmm.cpp:248-293: dx only.
+        dx = gmm_raw(grad[0], weight[0].transpose(-1, -2), group_list, 0, group_list_type or 0)
+        return [dx], [], []
+
+
+class _Builder:
+    _module = _RawGmmModule()
+
+    def load(self):
+        _lib.load()
+        return self._module
+
+
+def check_optional_tensor(tensor, device, name):
+    if not isinstance(tensor, (torch.Tensor, type(None))):
+        raise TypeError(f"{name} must be a torch.Tensor or None, got {type(tensor)}.")
+    if isinstance(tensor, torch.Tensor) and tensor.device != device:
+        raise RuntimeError(
+            f"Expected all tensors to be on the same device, but found at least two devices, "
+            f"{device}(arg0) and {tensor.device}({name})!")
+
+
+class GMMFunction(torch.autograd.Function):
+    builder = _Builder()
+    builder2 = _Builder()
+
+    @staticmethod
+    def forward(ctx, original_weight, x, weight, bias, group_args):
+        group_list, group_type, gemm_fusion, group_list_type, group_list_data_type = group_args
+        if bias is not None and bias.requires_grad:
+            raise ValueError("Bias is not supported to compute gradient!")
+        if (x.requires_grad or weight.requires_grad) and group_type != 0:
+            raise ValueError("group_type must be zero to compute gradients of x and weight!")
+        bias = [] if bias is None else [bias]
+        module = GMMFunction.builder.load() if group_list_type == 0 else GMMFunction.builder2.load()
+        outputs = module.npu_gmm([x], [weight], bias, group_list, group_type, group_list_type)
+        if group_list_data_type == 0:
+            ctx.save_for_backward(x, weight, original_weight)
+            ctx.group_list = group_list
+        else:
+            ctx.save_for_backward(x, weight, group_list, original_weight)
+        ctx.gemm_fusion = gemm_fusion
+        ctx.group_list_type = group_list_type
+        ctx.group_list_data_type = group_list_data_type
+        return outputs[0]
+
+    @staticmethod
+    def backward(ctx, grad_outputs):
+        if ctx.group_list_data_type == 0:
+            x, weight, original_weight = ctx.saved_tensors
+            group_list = ctx.group_list
+        else:
+            x, weight, group_list, original_weight = ctx.saved_tensors
+        module = GMMFunction.builder.load() if ctx.group_list_type == 0 else GMMFunction.builder2.load()
+
+        if ctx.gemm_fusion:
+            dx, _, dbias = module.npu_gmm_backward_fusion([grad_outputs], [weight], group_list, ctx.group_list_type)
+            if ctx.group_list_type == 0:
+                cumulative = group_list
+            else:
+                cumulative = torch.cumsum(group_list, dim=0)
+            npu_groupmatmul_add_fp32(x, grad_outputs, cumulative, original_weight.main_grad)
+            dbias = None if len(dbias) == 0 else dbias[0]
+            if hasattr(original_weight, "grad_added_to_main_grad"):
+                if getattr(weight, "zero_out_wgrad", False):
+                    grad_weight = torch.zeros(weight.shape, dtype=x.dtype, device=x.device, requires_grad=False)
+                else:
+                    grad_weight = torch.empty(weight.shape, dtype=x.dtype, device=x.device, requires_grad=False)
+                original_weight.grad_added_to_main_grad = True
+            else:
+                grad_weight = None
+            return None, dx[0], grad_weight, dbias, None
+
+        dx, dw, dbias = module.npu_gmm_backward([grad_outputs], [x], [weight], group_list, ctx.group_list_type)
+        dbias = None if len(dbias) == 0 else dbias[0]
+        return None, dx[0], dw[0], dbias, None
+
+
+def npu_gmm_param_verification(x, weight, *, bias=None, group_list=None, group_type=0, group_list_type=0):
+    if not isinstance(x, torch.Tensor):
+        raise TypeError(f"arg0 must be a torch.Tensor, got {type(x)}.")
+    if not isinstance(weight, torch.Tensor):
+        raise TypeError(f"arg1 must be a torch.Tensor, got {type(weight)}.")
+    if not isinstance(bias, (torch.Tensor, type(None))):
+        raise TypeError(f"bias must be a torch.Tensor or None, got {type(bias)}.")
+    if group_list_type == 0:
+        if not (
+            isinstance(group_list, (torch.Tensor, type(None)))
+            or (isinstance(group_list, list) and all(isinstance(v, int) for v in group_list))
+        ):
+            raise TypeError(f"group_list must be a List of int64, torch.Tensor or None, got {type(group_list)}.")
+    else:
+        if not isinstance(group_list, (torch.Tensor, type(None))):
+            raise TypeError(f"group_list must be a torch.Tensor or None, got {type(group_list)}.")
+    if isinstance(group_list, torch.Tensor):
+        if len(group_list.shape) > 1:
+            raise ValueError(f"If group_list is not None, it must be an one-dimensional tensor, "
+                             f"got dimension of group_list: {len(group_list.shape)}!")
+        if group_list.dtype != torch.int64:
+            raise TypeError(f"group_list must be a List of int64, got group_list type: {type(group_list)}, "
+                            f"dtype: {group_list.dtype}!")
+    if not isinstance(group_type, (int, type(None))):
+        raise TypeError(f"group_type must be an int or None, got {type(group_type)}.")
+    x_device = x.device
+    device_warning = "Expected all tensors to be on the same device, but found at least two devices"
+    if weight.device != x_device:
+        raise RuntimeError(f"{device_warning}, {x_device}(arg0) and {weight.device}(arg1)!")
+    if bias is not None and bias.device != x_device:
+        raise RuntimeError(f"{device_warning}, {x_device}(arg0) and {bias.device}(bias)!")
+    if isinstance(group_list, torch.Tensor) and group_list.device != x_device:
+        raise RuntimeError(f"{device_warning}, {x_device}(arg0) and {group_list.device}(group_list)!")
+
+
+# --------------------------------------------------------------------------
+# dispatcher registration: same schemas as the reference, namespace "mindspeed"
+# --------------------------------------------------------------------------
+def _define_library():
+    try:
+        lib = torch.library.Library("mindspeed", "DEF")
+    except RuntimeError:
+        # another provider (the reference itself) already owns the namespace
+        lib = torch.library.Library("mindspeed", "FRAGMENT")
+    defined = []
+    for schema in (
+        "npu_gmm.List(Tensor? original_weight, Tensor x, Tensor weight, *, Tensor? bias=None, "
+        "int[]? group_list=None, int? group_type=0, bool? gemm_fusion=False) -> Tensor",
+        "npu_gmm.Tensor(Tensor? original_weight, Tensor x, Tensor weight, *, Tensor? bias=None, "
+        "Tensor? group_list=None, int? group_type=0, bool? gemm_fusion=False) -> Tensor",
+        "npu_gmm_v2.Tensor(Tensor? original_weight, Tensor x, Tensor weight, *, Tensor? bias=None, "
+        "Tensor? group_list=None, int? group_type=0, bool? gemm_fusion=False) -> Tensor",
+    ):
+        try:
+            lib.define(schema)
+            defined.append(schema.split("(")[0])
+        except RuntimeError:
+            pass
+    return lib, defined
+
+
+_LIBRARY, _DEFINED = _define_library()
+
+
+def _npu_gmm(original_weight, x, weight, *, bias=None, group_list=None, group_type=0, gemm_fusion=False):
+    group_list_data_type = 1 if isinstance(group_list, (torch.Tensor, type(None))) else 0
+    group_args = (group_list, group_type, gemm_fusion, 0, group_list_data_type)
+    return GMMFunction.apply(original_weight, x, weight, bias, group_args)
+
+
+def _npu_gmm_v2(original_weight, x, weight, *, bias=None, group_list=None, group_type=0, gemm_fusion=False):
+    group_args = (group_list, group_type, gemm_fusion, 1, 1)
+    return GMMFunction.apply(original_weight, x, weight, bias, group_args)
+
+
+for _name, _fn in (("npu_gmm.List", _npu_gmm), ("npu_gmm.Tensor", _npu_gmm), ("npu_gmm_v2.Tensor", _npu_gmm_v2)):
+    if _name in _DEFINED:
+        # The implementation is an autograd.Function over the raw kernel call,
+        # so it is registered as a composite that autograd sees through.
+        _LIBRARY.impl(_name, _fn, "CompositeImplicitAutograd")
+
+
+def _npu_gmm_common(original_weight, x, weight, *, bias=None, group_list=None, group_type=0, group_list_type=0,
+                    gemm_fusion=False):
+    support_dtype = [torch.float16, torch.bfloat16, torch.float32]
+    if isinstance(weight, torch.Tensor) and weight.dtype not in support_dtype:
+        raise TypeError(f"Only support non quant case, but got weight dtype {weight.dtype}.")
+    npu_gmm_param_verification(x, weight, bias=bias, group_list=group_list, group_type=group_type,
+                               group_list_type=group_list_type)
+    if group_list is None:
+        raise ValueError("group_list is required: the single-tensor (split_item=3) form needs group boundaries")
+    if bias is not None:
+        raise ValueError("bias is not supported by the grouped matmul kernels")
+    if group_list_type == 0:
+        return torch.ops.mindspeed.npu_gmm(original_weight, x, weight, bias=bias, group_list=group_list,
+                                           group_type=group_type, gemm_fusion=gemm_fusion)
+    elif group_list_type == 1:
+        return torch.ops.mindspeed.npu_gmm_v2(original_weight, x, weight, bias=bias, group_list=group_list,
+                                              group_type=group_type, gemm_fusion=gemm_fusion)
+    else:
+        raise ValueError(f"group_list_type must be 0 or 1, but got {group_list_type}.")
+
+
+def npu_gmm(x, weight, *, bias=None, group_list=None, group_type=0, gemm_fusion=False, original_weight=None):
+    """Grouped matmul; ``group_list`` holds cumulative row offsets (list or int64 tensor)."""
+    return _npu_gmm_common(original_weight, x, weight, bias=bias, group_list=group_list, group_type=group_type,
+                           group_list_type=0, gemm_fusion=gemm_fusion)
+
+
+def npu_gmm_v2(x, weight, *, bias=None, group_list=None, group_type=0, gemm_fusion=False, original_weight=None):
+    """Grouped matmul; ``group_list`` holds per-group row counts (int64 tensor)."""
+    return _npu_gmm_common(original_weight, x, weight, bias=bias, group_list=group_list, group_type=group_type,
+                           group_list_type=1, gemm_fusion=gemm_fusion)

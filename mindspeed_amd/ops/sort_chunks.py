@@ -1,0 +1,84 @@
+"""``sort_chunks_by_idxs`` on MI355X.
+
+Mirrors the dispatcher hook restated in mindspeed/core/transformer/moe/
+moe_feature/overlap/moe_common.py:377-398 (fused form:
+mindspeed/lite/ops/triton/sort_chunks_by_idx.py:300-348):
+``cat([split(input, split_sizes)[i] for i in sorted_idxs])``; the backward is
+the inverse row map.  ``split_sizes`` and ``sorted_idxs`` may be device
+tensors; nothing is read back to the host.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+__all__ = ["sort_chunks_by_idxs"]
+
+
+def _as_i64(v, device):
+    if isinstance(v, torch.Tensor):
+        return v.to(device=device, dtype=torch.int64).contiguous()
+    return torch.tensor(list(v), dtype=torch.int64, device=device)
+
+
+class _SortChunks(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, inp, split_sizes, sorted_idxs, probs):
+        lib = _lib.load()
+        _lib.require_device(inp, "input")
+        if inp.dim() != 2:
+            raise RuntimeError(f"input must be 2 dimensional, got {inp.dim()}-dimensional")
+        inp = inp.contiguous()
+        dev = inp.device
+        rows, hidden = inp.shape
+        out = torch.empty_like(inp)
+        row_map = torch.empty(rows, dtype=torch.int32, device=dev)
+        p = probs.contiguous() if probs is not None else None
+        out_p = torch.empty_like(p) if p is not None else None
+        if p is not None and p.numel() != rows:
+            raise RuntimeError(f"probs has {p.numel()} entries, expected {rows}")
+        with torch.cuda.device(dev):
+            _lib.check(lib.ms_sort_chunks(
+                _lib.stream_ptr(dev), _lib.ptr(inp), _lib.ptr(split_sizes), _lib.ptr(sorted_idxs),
+                split_sizes.numel(), rows, hidden, _lib.dtype_code(inp.dtype, "input"), _lib.ptr(p),
+                _lib.dtype_code(p.dtype, "probs") if p is not None else 0, _lib.ptr(out), _lib.ptr(out_p),
+                _lib.ptr(row_map)), "ms_sort_chunks")
+        ctx.save_for_backward(row_map)
+        ctx.has_probs = p is not None
+        ctx.mark_non_differentiable(row_map)
+        if p is None:
+            return out, None, row_map
+        return out, out_p, row_map
+
+    @staticmethod
+    def backward(ctx, grad_out, grad_probs, _grad_map):
+        (row_map,) = ctx.saved_tensors
+        lib = _lib.load()
+        dev = grad_out.device
+        g = grad_out.contiguous()
+        gi = torch.empty_like(g)
+        with torch.cuda.device(dev):
+            _lib.check(lib.ms_gather_rows(_lib.stream_ptr(dev), _lib.ptr(g), _lib.ptr(row_map), g.size(0), g.size(1),
+                                          _lib.dtype_code(g.dtype, "grad"), 1, _lib.ptr(gi)), "ms_gather_rows")
+        gp = None
+        if ctx.has_probs and grad_probs is not None:
+            gpc = grad_probs.contiguous()
+            gp = torch.empty_like(gpc)
+            with torch.cuda.device(dev):
+                _lib.check(lib.ms_gather_rows(_lib.stream_ptr(dev), _lib.ptr(gpc), _lib.ptr(row_map), gpc.numel(), 1,
+                                              _lib.dtype_code(gpc.dtype, "grad_probs"), 1, _lib.ptr(gp)),
+                           "ms_gather_rows")
+        return gi, None, None, gp
+
+
+def sort_chunks_by_idxs(input, split_sizes, sorted_idxs, probs=None, fused=True):
+    """Returns ``(output, permuted_probs)`` like the reference hook."""
+    del fused  # one code path
+    dev = input.device
+    split_sizes = _as_i64(split_sizes, dev)
+    sorted_idxs = _as_i64(sorted_idxs, dev)
+    if split_sizes.numel() != sorted_idxs.numel():
+        raise RuntimeError("split_sizes and sorted_idxs must have the same length")
+    out, out_probs, _ = _SortChunks.apply(input, split_sizes, sorted_idxs, probs)
+    return out, out_probs

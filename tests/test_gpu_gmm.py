@@ -1,0 +1,204 @@
+"""GPU parity: grouped matmul forward, dX, dW and the fp32 accumulate form
+against the CPU oracle and the integer golden fixtures, through the Python
+surface that calls the C ABI.  Tolerance: rel-L2 <= 1e-2 for bf16 / fp16,
+<= 1e-5 for fp32; integer-valued fixtures must match exactly."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import rel_l2
+from oracle import moe_oracle as O
+
+import mindspeed_amd.ops as ops
+from mindspeed_amd.ops.gmm import gmm_raw
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+TOL = {torch.bfloat16: 1e-2, torch.float16: 1e-2, torch.float32: 1e-5}
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_reference_test_shapes_exact(dtype, device):
+    """Shapes / group lists of the reference's own unit test, on integers: exact in every dtype."""
+    g = np.load(os.path.join(GOLDEN, "gmm_cases.npz"))
+    for name in ("rows_a", "rows_b", "rows_doc"):
+        say("golden", name, dtype)
+        counts = g[f"{name}_counts"].tolist()
+        x = torch.from_numpy(g[f"{name}_x"]).to(dtype).to(device)
+        w = torch.from_numpy(g[f"{name}_w"]).to(dtype).to(device)
+        y = torch.from_numpy(g[f"{name}_y"]).float()
+        cum = np.cumsum(counts).tolist()
+        assert torch.equal(ops.npu_gmm(x, w, bias=None, group_list=cum, group_type=0).float().cpu(), y)
+        assert torch.equal(ops.npu_gmm(x, w, group_list=torch.tensor(cum, device=device), group_type=0).float().cpu(), y)
+        assert torch.equal(ops.npu_gmm_v2(x, w, group_list=torch.tensor(counts, device=device), group_type=0).float().cpu(), y)
+    for name in ("red_a", "red_empty"):
+        say("golden", name, dtype)
+        counts = g[f"{name}_counts"].tolist()
+        x = torch.from_numpy(g[f"{name}_x"]).to(dtype).to(device)      # [M, 48]; the op sees x.T
+        w = torch.from_numpy(g[f"{name}_w"]).to(dtype).to(device)
+        y = torch.from_numpy(g[f"{name}_y"]).float()
+        got = ops.npu_gmm_v2(x.t(), w, group_list=torch.tensor(counts, device=device), group_type=2)
+        assert got.shape == y.shape and torch.equal(got.float().cpu(), y)
+        got = ops.npu_gmm(x.t(), w, group_list=np.cumsum(counts).tolist(), group_type=2)
+        assert torch.equal(got.float().cpu(), y)
+
+
+def test_groupmatmul_add_fixture(device):
+    g = np.load(os.path.join(GOLDEN, "groupmatmul_add.npz"))
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        say("groupmatmul_add golden", dtype)
+        x = torch.from_numpy(g["x"]).to(dtype).to(device)
+        dy = torch.from_numpy(g["dy"]).to(dtype).to(device)
+        acc = torch.from_numpy(g["acc"]).float().to(device)
+        ops.npu_groupmatmul_add_fp32(x, dy, torch.from_numpy(g["offsets"]).to(device), acc)
+        assert torch.equal(acc.cpu(), torch.from_numpy(g["expect"]).float())
+
+
+def _counts(kind, E, M, seed):
+    gen = torch.Generator().manual_seed(seed)
+    if kind == "equal":
+        c = torch.full((E,), M // E)
+        c[-1] += M - c.sum()
+    elif kind == "skew_empty":                     # Zipf-like skew with one empty group
+        w = 1.0 / torch.arange(1, E + 1).float() ** 1.2
+        w = w[torch.randperm(E, generator=gen)]
+        w[int(torch.randint(0, E, (1,), generator=gen))] = 0
+        c = torch.floor(w / w.sum() * M).long()
+        c[int(torch.argmax(c))] += M - c.sum()
+    else:                                          # random, several empty
+        cuts = torch.sort(torch.randint(0, M + 1, (E - 1,), generator=gen))[0]
+        c = torch.diff(torch.cat([torch.tensor([0]), cuts, torch.tensor([M])]))
+    assert c.sum() == M and (c >= 0).all()
+    return c.long()
+
+
+GMM_CASES = [
+    # M, K, N, E, kind
+    (1024, 256, 1024, 8, "random"),
+    (1000, 200, 328, 8, "random"),        # nothing a multiple of the tile
+    (513, 72, 40, 3, "skew_empty"),
+    (4096, 512, 768, 8, "skew_empty"),
+    (2048, 128, 512, 64, "random"),       # many small groups, several < 64 rows
+    (300, 64, 256, 1, "equal"),
+    (96, 1000, 24, 4, "equal"),           # long reduction, narrow output
+    (37, 19, 23, 5, "random"),            # tiny and odd: element-wise paths
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,K,N,E,kind", GMM_CASES)
+def test_forward_and_backward_vs_oracle(M, K, N, E, kind, dtype, device):
+    say("gmm case", M, K, N, E, kind, dtype)
+    gen = torch.Generator().manual_seed(M + K + N)
+    counts = _counts(kind, E, M, seed=M)
+    x = torch.randn(M, K, generator=gen).to(dtype)
+    w = (torch.randn(E, K, N, generator=gen) * 0.05).to(dtype)
+    gy = torch.randn(M, N, generator=gen).to(dtype)
+    exp_y = O.gmm(x, w, counts, 0, 1)
+    exp_dx, exp_dw = O.gmm_backward(gy, x, w, counts, 1)
+
+    xd = x.to(device).requires_grad_(True)
+    wd = w.to(device).requires_grad_(True)
+    y = ops.npu_gmm_v2(xd, wd, group_list=counts.to(device), group_type=0)
+    y.backward(gy.to(device))
+    torch.cuda.synchronize()
+    tol = TOL[dtype]
+    assert y.shape == (M, N) and rel_l2(y, exp_y) <= tol
+    assert rel_l2(xd.grad, exp_dx) <= tol
+    assert wd.grad.shape == w.shape and rel_l2(wd.grad, exp_dw) <= tol
+    for gidx in torch.nonzero(counts == 0).flatten().tolist():
+        assert torch.count_nonzero(wd.grad[gidx]) == 0          # empty group => zero dW block
+    # fp64 bound
+    y64 = O.gmm(x.double(), w.double(), counts, 0, 1)
+    assert rel_l2(y, y64) <= tol
+    # cumulative list form gives the same bits
+    y2 = ops.npu_gmm(x.to(device), w.to(device), group_list=torch.cumsum(counts, 0).tolist(), group_type=0)
+    assert torch.equal(y2, y.detach())
+
+
+def test_transposed_weight_view_and_raw_module(device):
+    """A weight stored [E, N, K] and passed as .transpose(1, 2) (Ops.gmm's trans_b form) needs no copy."""
+    gen = torch.Generator().manual_seed(5)
+    M, K, N, E = 700, 192, 320, 4
+    counts = _counts("random", E, M, 5)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    wt = (torch.randn(E, N, K, generator=gen) * 0.05).to(torch.bfloat16)
+    exp = O.gmm(x, wt.transpose(1, 2), counts, 0, 1)
+    got = ops.npu_gmm_v2(x.to(device), wt.to(device).transpose(1, 2), group_list=counts.to(device))
+    assert rel_l2(got, exp) <= 1e-2
+    # raw list-in / list-out module used by BaseGMMFunction subclasses
+    mod = ops.GMMFunction.builder.load()
+    cum = torch.cumsum(counts, 0).to(device)
+    w = wt.transpose(1, 2).contiguous().to(device)
+    (y,) = mod.npu_gmm([x.to(device)], [w], [], cum, 0, 0)
+    gy = torch.randn(M, N, generator=gen).to(torch.bfloat16)
+    dx, dw, dbias = mod.npu_gmm_backward([gy.to(device)], [x.to(device)], [w], cum, 0)
+    e_dx, e_dw = O.gmm_backward(gy, x, w.cpu(), counts, 1)
+    assert rel_l2(y, exp) <= 1e-2 and rel_l2(dx[0], e_dx) <= 1e-2 and rel_l2(dw[0], e_dw) <= 1e-2 and dbias == []
+    dx2, dw2, _ = mod.npu_gmm_backward_fusion([gy.to(device)], [w], cum, 0)
+    assert torch.equal(dx2[0], dx[0]) and dw2 == []
+
+
+def test_rows_past_last_offset_are_zero(device):
+    gen = torch.Generator().manual_seed(6)
+    x = torch.randn(600, 64, generator=gen).to(torch.bfloat16).to(device)
+    w = torch.randn(3, 64, 96, generator=gen).to(torch.bfloat16).to(device)
+    y = ops.npu_gmm(x, w, group_list=[100, 100, 430], group_type=0)
+    exp = O.gmm(x.cpu(), w.cpu(), [100, 100, 430], 0, 0)
+    assert torch.count_nonzero(y[430:]) == 0 and rel_l2(y, exp) <= 1e-2
+
+
+def test_gemm_fusion_accumulates_into_main_grad(device):
+    """gemm_fusion=True: dW is added into original_weight.main_grad (fp32) and a dummy grad is returned
+    (mindspeed/ops/gmm.py:56-89)."""
+    gen = torch.Generator().manual_seed(8)
+    M, K, N, E = 512, 96, 160, 4
+    counts = _counts("skew_empty", E, M, 8)
+    cum = torch.cumsum(counts, 0)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(E, K, N, generator=gen) * 0.05).to(torch.bfloat16)
+    gy = torch.randn(M, N, generator=gen).to(torch.bfloat16)
+    main0 = torch.randn(E * K, N, generator=gen)
+    param = torch.nn.Parameter(w.to(device))
+    param.main_grad = main0.clone().to(device)
+    param.grad_added_to_main_grad = False
+    xd = x.to(device).requires_grad_(True)
+    y = ops.npu_gmm(xd, param, group_list=cum.to(device), group_type=0, gemm_fusion=True, original_weight=param)
+    y.backward(gy.to(device))
+    exp_dx, _ = O.gmm_backward(gy, x, w, counts, 1)
+    exp_main = O.groupmatmul_add_fp32(x, gy, cum, main0.clone())
+    assert param.grad_added_to_main_grad is True
+    assert rel_l2(xd.grad, exp_dx) <= 1e-2
+    assert rel_l2(param.main_grad, exp_main) <= 1e-5
+    # v2 (counts) form
+    param.main_grad = main0.clone().to(device)
+    xd2 = x.to(device).requires_grad_(True)
+    ops.npu_gmm_v2(xd2, param, group_list=counts.to(device), gemm_fusion=True, original_weight=param).backward(gy.to(device))
+    assert rel_l2(param.main_grad, exp_main) <= 1e-5
+
+
+def test_linearity_at_mixtral_fc1_shape(device):
+    """Full-size property check on the Mixtral fc1 shape: gmm(a*x1 + x2) == a*gmm(x1) + gmm(x2) within bf16
+    rounding, and sampled rows against per-row fp32 matmuls."""
+    T, H, F, E = 8192, 4096, 14336, 8
+    say("mixtral fc1 linearity")
+    gen = torch.Generator(device=device).manual_seed(0)
+    w = (torch.randn(E, H, 2 * F, generator=gen, device=device) * 0.02).to(torch.bfloat16)
+    x1 = torch.randn(T, H, generator=gen, device=device).to(torch.bfloat16)
+    counts = torch.tensor([1100, 900, 1024, 1024, 1200, 848, 1000, 1096], device=device)
+    y1 = ops.npu_gmm_v2(x1, w, group_list=counts)
+    y2 = ops.npu_gmm_v2(x1 * 2, w, group_list=counts)                 # exact scaling in bf16
+    assert torch.equal(y2, y1 * 2)
+    rows = torch.randint(0, T, (48,), generator=torch.Generator().manual_seed(1))
+    bounds = torch.cumsum(counts.cpu(), 0)
+    for r in rows.tolist():
+        g = int(torch.searchsorted(bounds, torch.tensor(r), right=True))
+        ref = x1[r].float().cpu() @ w[g].float().cpu()
+        assert rel_l2(y1[r], ref) <= 1e-2, r

@@ -1,0 +1,116 @@
+"""Host-side mirror of the reference interface: signatures, argument checks and
+error types, and the rule that nothing computes off the GPU.  No GPU needed."""
+import inspect
+
+import pytest
+import torch
+
+import mindspeed_amd.ops as ops
+from mindspeed_amd.ops import gmm as gmm_mod
+
+
+def test_signatures_match_reference():
+    # mindspeed/ops/npu_moe_token_permute.py:13-18
+    assert list(inspect.signature(ops.npu_moe_token_permute).parameters) == [
+        "tokens", "indices", "num_out_tokens", "padded_mode"]
+    # mindspeed/ops/npu_moe_token_unpermute.py:13-19
+    assert list(inspect.signature(ops.npu_moe_token_unpermute).parameters) == [
+        "permuted_tokens", "sorted_indices", "probs", "padded_mode", "restore_shape"]
+    # mindspeed/ops/gmm.py:164,174
+    for fn in (ops.npu_gmm, ops.npu_gmm_v2):
+        sig = inspect.signature(fn)
+        assert list(sig.parameters) == ["x", "weight", "bias", "group_list", "group_type", "gemm_fusion",
+                                        "original_weight"]
+        assert all(sig.parameters[p].kind is inspect.Parameter.KEYWORD_ONLY for p in list(sig.parameters)[2:])
+    # mindspeed/ops/npu_groupmatmul_add.py:11
+    assert list(inspect.signature(ops.npu_groupmatmul_add_fp32).parameters) == ["x", "dy", "grouplist", "grad"]
+
+
+def test_dispatcher_schemas_registered():
+    assert hasattr(torch.ops.mindspeed, "npu_gmm") and hasattr(torch.ops.mindspeed, "npu_gmm_v2")
+    assert {"List", "Tensor"} <= set(torch.ops.mindspeed.npu_gmm.overloads())
+    assert "Tensor" in torch.ops.mindspeed.npu_gmm_v2.overloads()
+
+
+def test_no_cpu_fallback():
+    x = torch.randn(8, 16, dtype=torch.bfloat16)
+    idx = torch.zeros(8, 2, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.npu_moe_token_permute(x, idx)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.npu_moe_token_unpermute(x, torch.zeros(8, dtype=torch.int32))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.npu_gmm(x, torch.randn(2, 16, 4, dtype=torch.bfloat16), group_list=[4, 8])
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.fused_swiglu(x)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.sort_chunks_by_idxs(x, [4, 4], [1, 0])
+
+
+def test_permute_argument_checks():
+    x = torch.randn(8, 16, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="padded_mode"):
+        ops.npu_moe_token_permute(x, torch.zeros(8, 2, dtype=torch.int64), padded_mode=True)
+    with pytest.raises(TypeError, match="int64 or int32"):
+        ops.npu_moe_token_permute(x, torch.zeros(8, 2, dtype=torch.int16))
+    with pytest.raises(TypeError, match="tokens"):
+        ops.npu_moe_token_permute(x.to(torch.float64), torch.zeros(8, 2, dtype=torch.int64))
+    with pytest.raises(RuntimeError, match="2 dimensional"):
+        ops.npu_moe_token_permute(x.view(2, 4, 16), torch.zeros(8, 2, dtype=torch.int64))
+    with pytest.raises(RuntimeError, match="2 or 1 dimensional"):
+        ops.npu_moe_token_permute(x, torch.zeros(8, 2, 1, dtype=torch.int64))
+
+
+def test_unpermute_argument_checks():
+    x = torch.randn(8, 16, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="padded_mode"):
+        ops.npu_moe_token_unpermute(x, torch.zeros(8, dtype=torch.int32), padded_mode=True)
+    with pytest.raises(TypeError, match="int32"):
+        ops.npu_moe_token_unpermute(x, torch.zeros(8, dtype=torch.int64))
+    with pytest.raises(RuntimeError, match="1 dimensional"):
+        ops.npu_moe_token_unpermute(x, torch.zeros(4, 2, dtype=torch.int32))
+    with pytest.raises(RuntimeError, match="probs should be 2 dimensional"):
+        ops.npu_moe_token_unpermute(x, torch.zeros(8, dtype=torch.int32), torch.ones(8, dtype=torch.bfloat16))
+
+
+def test_gmm_argument_checks():
+    # mindspeed/ops/gmm.py:103-150
+    x = torch.randn(8, 16, dtype=torch.bfloat16)
+    w = torch.randn(2, 16, 4, dtype=torch.bfloat16)
+    with pytest.raises(TypeError, match="arg0"):
+        ops.npu_gmm([1], w, group_list=[4, 8])
+    with pytest.raises(TypeError, match="arg1"):
+        ops.npu_gmm(x, None, group_list=[4, 8])
+    with pytest.raises(TypeError, match="bias"):
+        ops.npu_gmm(x, w, bias=3, group_list=[4, 8])
+    with pytest.raises(TypeError, match="group_list must be a List of int64, torch.Tensor or None"):
+        ops.npu_gmm(x, w, group_list=(4, 8))
+    with pytest.raises(TypeError, match="group_list must be a torch.Tensor or None"):
+        ops.npu_gmm_v2(x, w, group_list=[4, 4])
+    with pytest.raises(ValueError, match="one-dimensional"):
+        ops.npu_gmm(x, w, group_list=torch.zeros(2, 2, dtype=torch.int64))
+    with pytest.raises(TypeError, match="dtype"):
+        ops.npu_gmm(x, w, group_list=torch.zeros(2, dtype=torch.int32))
+    with pytest.raises(TypeError, match="group_type"):
+        ops.npu_gmm(x, w, group_list=[4, 8], group_type="0")
+    with pytest.raises(TypeError, match="non quant"):
+        ops.npu_gmm(x, w.to(torch.int8), group_list=[4, 8])
+    with pytest.raises(ValueError, match="group_list_type"):
+        gmm_mod._npu_gmm_common(None, x, w, group_list=torch.tensor([4, 8]), group_list_type=3)
+
+
+def test_raw_module_surface():
+    # mindspeed/ops/csrc/cann/gmm.cpp:295-309
+    mod = ops.GMMFunction.builder.load()
+    for name in ("npu_gmm", "npu_gmm_backward", "npu_gmm_backward_fusion"):
+        assert callable(getattr(mod, name))
+    assert callable(getattr(ops.GMMFunction.builder2.load(), "npu_gmm"))
+
+
+def test_groupmatmul_add_checks():
+    x = torch.randn(8, 16, dtype=torch.bfloat16)
+    dy = torch.randn(8, 4, dtype=torch.bfloat16)
+    with pytest.raises(TypeError, match="float32"):
+        ops.npu_groupmatmul_add_fp32(x, dy, torch.tensor([4, 8]), torch.zeros(32, 4, dtype=torch.bfloat16))
+    with pytest.raises(ValueError, match="elements"):
+        ops.npu_groupmatmul_add_fp32(x, dy, torch.tensor([4, 8]), torch.zeros(31, 4))
