@@ -1,0 +1,204 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-rank MoE expert path on one MI355X.
+
+A step is one forward + backward pass of a single MoE layer (permute, grouped
+matmul, SiLU*gate, grouped matmul, weighted unpermute, and all their
+gradients) over one batch of synthetic tokens that is resident in HBM before
+the timed region starts.  The default workload is the Mixtral-8x7B-shape layer
+(4096 tokens, hidden 4096, 8 experts, top-2, FFN 14336, bf16, fp32
+accumulation).  One JSON line is printed.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixtral|deepseek|qwen|plumbing]
+                    [--no-cpu-baseline]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}   # dense, published
+
+WORKLOADS = {
+    # name: (tokens, hidden, experts, topk, ffn, dtype, routing)
+    "plumbing": dict(T=512, H=256, E=8, K=2, F=512, dtype="f32", routing="uniform",
+                     desc="configs[0]: 512 tokens, hidden 256, 8 experts, top-2, ffn 512, fp32"),
+    "mixtral": dict(T=4096, H=4096, E=8, K=2, F=14336, dtype="bf16", routing="uniform",
+                    desc="configs[1]/[2] Mixtral-8x7B-shape MoE layer: 4096 tokens, hidden 4096, 8 experts, "
+                         "top-2, ffn 14336, bf16, forward+backward"),
+    "deepseek": dict(T=2048, H=7168, E=8, K=8, F=2048, dtype="bf16", routing="zipf_empty",
+                     desc="configs[3] DeepSeek-V3-style local share: 16384 rows, hidden 7168, 8 local experts, "
+                          "ffn 2048, Zipf(1.2) with one empty expert, bf16, forward+backward"),
+    "qwen": dict(T=8192, H=2048, E=64, K=8, F=1408, dtype="bf16", routing="biased",
+                 desc="configs[4] fine-grained MoE: 8192 tokens, hidden 2048, 64 experts, top-8, ffn 1408, "
+                      "biased routing, bf16, forward+backward"),
+}
+
+
+def make_routing(cfg, seed=0):
+    """Routing indices / probabilities on the CPU (deterministic), per the workload's recipe."""
+    gen = torch.Generator().manual_seed(seed)
+    T, E, K = cfg["T"], cfg["E"], cfg["K"]
+    if cfg["routing"] == "zipf_empty":
+        pmf = 1.0 / torch.arange(1, E + 1, dtype=torch.float64) ** 1.2
+        pmf = pmf[torch.randperm(E, generator=gen)]
+        empty = int(torch.randint(0, E, (1,), generator=gen))
+        idx = torch.multinomial(pmf / pmf.sum(), T * K, replacement=True, generator=gen)
+        idx[idx == empty] = (empty + 1) % E
+        idx = idx.view(T, K)
+        probs = torch.distributions.Dirichlet(torch.ones(K)).sample((T,))
+        return probs.float(), idx
+    logits = torch.randn(T, E, generator=gen)
+    if cfg["routing"] == "biased":
+        logits = logits + 1.5 * torch.randn(E, generator=gen)
+    full = torch.softmax(logits, dim=-1)
+    p, idx = torch.topk(full, K, dim=-1)
+    return (p / p.sum(-1, keepdim=True)).float(), idx
+
+
+def make_inputs(cfg, device, seed=0):
+    dtype = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+    T, H, E, F = cfg["T"], cfg["H"], cfg["E"], cfg["F"]
+    gen = torch.Generator(device=device).manual_seed(seed)
+    x = torch.randn(T, H, generator=gen, device=device).to(dtype)
+    w1 = (torch.randn(E, H, 2 * F, generator=gen, device=device) * 0.02).to(dtype)
+    w2 = (torch.randn(E, F, H, generator=gen, device=device) * 0.02).to(dtype)
+    gy = torch.randn(T, H, generator=gen, device=device).to(dtype)
+    p, idx = make_routing(cfg, seed)
+    return x, p.to(dtype).to(device), idx.to(device), w1, w2, gy
+
+
+def _cpu_layer_once(cfg, sample):
+    from oracle import moe_oracle as O
+
+    T, H, E, K, F = cfg["T"], cfg["H"], cfg["E"], cfg["K"], cfg["F"]
+    sub = dict(cfg, T=sample)
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(sample, H, generator=gen).requires_grad_(True)
+    w1 = (torch.randn(E, H, 2 * F, generator=gen) * 0.02).requires_grad_(True)
+    w2 = (torch.randn(E, F, H, generator=gen) * 0.02).requires_grad_(True)
+    gy = torch.randn(sample, H, generator=gen)
+    p, idx = make_routing(sub, 0)
+    p = p.requires_grad_(True)
+    t0 = time.perf_counter()
+    out = O.moe_layer(x, idx, p, w1, w2)
+    torch.autograd.grad(out, (x, p, w1, w2), gy)
+    return time.perf_counter() - t0
+
+
+def cpu_baseline(cfg, budget_s=15.0):
+    """The CPU oracle (torch restatement of the reference's pure-PyTorch path) timed on this host, fp32,
+    forward + backward, on a token sample sized (from a short probe run) to about budget_s of CPU work."""
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    T = cfg["T"]
+    probe = min(T, 128)
+    t_probe = _cpu_layer_once(cfg, probe)          # also warms the thread pool
+    sample = int(min(T, max(probe, probe * budget_s / max(t_probe, 1e-3))))
+    sample = max(64, (sample // 64) * 64) if sample >= 64 else sample
+    dt = _cpu_layer_once(cfg, sample) if sample != probe else _cpu_layer_once(cfg, probe)
+    return {"value": round(sample / dt, 2), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"{sample} of {T} tokens, same layer shape, fp32, one forward+backward "
+                      f"({dt:.1f} s) with torch {torch.__version__} on {threads} threads"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="mixtral", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py measures one rank's expert path on ONE GPU (no collectives are part of this path); "
+                 "run it with --gpus 1.")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a HIP device")
+
+    from mindspeed_amd import flop_counter
+    from mindspeed_amd.dispatcher import dispatch_mlp_combine
+
+    cfg = WORKLOADS[args.workload]
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    x, p, idx, w1, w2, gy = make_inputs(cfg, device)
+    leaves = [t.requires_grad_(True) for t in (x, p, w1, w2)]
+
+    def step():
+        out = dispatch_mlp_combine(leaves[0], idx, leaves[1], (leaves[2], leaves[3]))
+        return torch.autograd.grad(out, leaves, gy)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    with flop_counter.record(timing=True) as rec:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    tokens_per_s = cfg["T"] / (ms_per_step / 1e3)
+
+    # per-op breakdown from the events recorded on the launch stream inside the timed region
+    kernels = {}
+    for name, s in rec.summary().items():
+        avg_ms = s["ms"] / s["calls"]
+        work = s["work"] / s["calls"]
+        entry = {"calls_per_step": s["calls"] / args.steps, "avg_ms": round(avg_ms, 5)}
+        if s["unit"] == "flop":
+            entry["tflops"] = round(work / (avg_ms * 1e-3) / 1e12, 2)
+            entry["flop_per_launch"] = work
+        else:
+            entry["gbs"] = round(work / (avg_ms * 1e-3) / 1e9, 1)
+            entry["bytes_per_launch"] = work
+        kernels[name] = entry
+
+    peak = MFMA_PEAK_TFLOPS[cfg["dtype"]]
+    dom = kernels["gmm_fwd"]          # the forward grouped matmul: fc1 and fc2 launches averaged
+    roofline = {"bound": "mfma", "kernel": "gmm16_kernel (NN, forward grouped matmul; fc1+fc2 averaged)"
+                if cfg["dtype"] == "bf16" else "gmm32_kernel", "achieved": dom["tflops"], "peak": peak,
+                "unit": "TFLOP/s", "frac": round(dom["tflops"] / peak, 4), "traffic": None}
+    for name in ("gmm_dx", "gmm_dw"):
+        kernels[name]["frac_of_mfma_peak"] = round(kernels[name]["tflops"] / peak, 4)
+    kernels["gmm_fwd"]["frac_of_mfma_peak"] = roofline["frac"]
+    for name, e in kernels.items():
+        if "gbs" in e:
+            e["frac_of_hbm_peak"] = round(e["gbs"] / HBM_PEAK_GBS, 4)
+
+    result = {
+        "metric": "MoE layer fwd+bwd tokens/s at 1 GPU",
+        "value": round(tokens_per_s, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": cfg["dtype"],
+        "data": "synthetic",
+        "config": {"workload": cfg["desc"], "tokens": cfg["T"], "hidden": cfg["H"], "experts": cfg["E"],
+                   "topk": cfg["K"], "ffn": cfg["F"], "gemm_tflop_per_step": round(18.0 * cfg["T"] * cfg["K"]
+                                                                                  * cfg["H"] * cfg["F"] / 1e12, 3)},
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(cfg)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

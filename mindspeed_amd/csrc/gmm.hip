@@ -19,46 +19,10 @@
 //     panel, so concurrently running workgroups of an XCD share weight panels
 //     in that XCD's L2.
 //   * gmm32_kernel: fp32 inputs, v_mfma_f32_32x32x2f32, 128x128x8 tiles.
-#include "common.h"
+#include "gmm_common.h"
 
 namespace ms {
 namespace {
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-constexpr int kMaxGroups = 4096;
-
-struct GroupEntry {
-    int row_begin, row_end;  // output rows of the group
-    int red_begin, red_end;  // reduction range of the group
-    int tile_begin;          // first logical tile
-    int num_row_tiles;
-    int64_t b_off;           // element offset of the group's weight block
-    int64_t c_off;           // element offset of the group's output block
-};
-
-struct TileTable {
-    int total_tiles;
-    int num_entries;
-    int pad[6];
-    GroupEntry entries[1];
-};
-
-struct GmmArgs {
-    const void *a;
-    const void *b;
-    void *c;
-    const TileTable *table;
-    int64_t a_stride_row, a_stride_red;
-    int64_t b_stride_red, b_stride_col;
-    int64_t c_stride_row;
-    int cols;          // n
-    int num_col_tiles;
-    int a_vec_ok, b_vec_ok, c_vec_ok;
-};
 
 // ---- schedule ------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__restrict__ group_list,
@@ -116,54 +80,7 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
     table->num_entries = n;
 }
 
-struct TileCoord {
-    GroupEntry e;
-    int row_tile, col_tile;
-    bool valid;
-};
-
-// Map this workgroup to its logical tile (XCD-aware, see file header).
-__device__ __forceinline__ TileCoord locate_tile(const TileTable *table) {
-    TileCoord tc;
-    tc.valid = false;
-    const int total = table->total_tiles;
-    const int per_xcd = (total + 7) >> 3;
-    const int xcd = blockIdx.x & 7;
-    const int slot = blockIdx.x >> 3;
-    if (slot >= per_xcd) return tc;
-    const int logical = xcd * per_xcd + slot;
-    if (logical >= total) return tc;
-    int lo = 0, hi = table->num_entries;  // last entry with tile_begin <= logical
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (table->entries[mid].tile_begin <= logical) lo = mid; else hi = mid;
-    }
-    tc.e = table->entries[lo];
-    const int r = logical - tc.e.tile_begin;
-    tc.col_tile = r / tc.e.num_row_tiles;
-    tc.row_tile = r - tc.col_tile * tc.e.num_row_tiles;
-    tc.valid = true;
-    return tc;
-}
-
 // ---- 16-bit MFMA kernel ------------------------------------------------------------------
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kTileBytes = BM * BK * 2;                 // 32 KB per operand per stage
-constexpr int kLdsBytes16 = 4 * kTileBytes;             // A,B x 2 stages = 128 KB
-
-enum OutMode { OUT_SAME = 0, OUT_F32 = 1, ACC_F32 = 2 };
-
-template <int DT>
-__device__ __forceinline__ f32x16 mfma16(v16 a, v16 b, f32x16 c) {
-    if constexpr (DT == MS_BF16) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
-                                                       0, 0, 0);
-    } else {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
-                                                      0, 0);
-    }
-}
-
 // 8 contiguous 16-bit elements starting at p; elements >= nvalid read as zero.
 __device__ __forceinline__ v16 load8(const uint16_t *p, int nvalid, bool vec_ok) {
     if (nvalid >= 8 && vec_ok && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) return *reinterpret_cast<const v16 *>(p);
@@ -176,9 +93,6 @@ __device__ __forceinline__ v16 load8(const uint16_t *p, int nvalid, bool vec_ok)
     }
     return r;
 }
-
-// LDS swizzle: 16-byte chunk position of (row, chunk) inside the row's 128 bytes.
-__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
 // Operand tile loader.  RED == true: memory is contiguous along the reduction
 // dim; RED == false: contiguous along the outer (row of A / col of B) dim.
@@ -594,6 +508,20 @@ extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int
     if (!use_b_red && b_stride_col != 1) args.b_vec_ok = 0;
 
     const int out = accumulate ? ACC_F32 : (out_dtype == MS_FP32 ? OUT_F32 : OUT_SAME);
+    // The fast kernels need 16-byte vector access everywhere: aligned bases, strides in multiples of 8
+    // elements, whole 8-element chunks along every contiguous dim, and (for operands contiguous along the
+    // reduction dim) reduction ranges that start at multiples of 8, i.e. no split on the reduction dim.
+    const bool a_truly_contig = a_is_red ? a_stride_red == 1 : a_stride_row == 1;
+    const bool b_truly_contig = b_is_red ? b_stride_red == 1 : b_stride_col == 1;
+    bool fast = args.a_vec_ok && args.b_vec_ok && args.c_vec_ok && a_truly_contig && b_truly_contig;
+    if (a_is_red) fast = fast && red_total % 8 == 0 && group_type == 0; else fast = fast && out_rows % 8 == 0 && out_rows >= 8;
+    if (b_is_red) fast = fast && red_total % 8 == 0 && group_type == 0; else fast = fast && n % 8 == 0 && n >= 8;
+    fast = fast && n % 4 == 0 && (out_dtype != MS_FP32 || reinterpret_cast<uintptr_t>(y) % 16 == 0);
+    // per-lane global offsets are 32-bit byte offsets inside one 256 x 64 operand tile
+    const int64_t a_span = a_is_red ? 256 * a_stride_row : 64 * a_stride_red;
+    const int64_t b_span = b_is_red ? 256 * b_stride_col : 64 * b_stride_red;
+    fast = fast && a_span < (1ll << 30) && b_span < (1ll << 30);
+    if (fast) return launch_gmm16_fast(stream, args, dtype, out, a_is_red, b_is_red, grid);
     if (dtype == MS_BF16) {
         if (out == OUT_SAME) return launch16<MS_BF16, OUT_SAME>(stream, args, a_is_red, b_is_red, grid);
         if (out == OUT_F32) return launch16<MS_BF16, OUT_F32>(stream, args, a_is_red, b_is_red, grid);

@@ -1,0 +1,100 @@
+// Declarations shared by the grouped-matmul translation units.
+#pragma once
+
+#include "common.h"
+
+namespace ms {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kMaxGroups = 4096;
+
+struct GroupEntry {
+    int row_begin, row_end;  // output rows of the group
+    int red_begin, red_end;  // reduction range of the group
+    int tile_begin;          // first logical tile
+    int num_row_tiles;
+    int64_t b_off;           // element offset of the group's weight block
+    int64_t c_off;           // element offset of the group's output block
+};
+
+struct TileTable {
+    int total_tiles;
+    int num_entries;
+    int pad[6];
+    GroupEntry entries[1];
+};
+
+struct GmmArgs {
+    const void *a;
+    const void *b;
+    void *c;
+    const TileTable *table;
+    int64_t a_stride_row, a_stride_red;
+    int64_t b_stride_red, b_stride_col;
+    int64_t c_stride_row;
+    int cols;          // n
+    int num_col_tiles;
+    int a_vec_ok, b_vec_ok, c_vec_ok;
+};
+
+struct TileCoord {
+    GroupEntry e;
+    int row_tile, col_tile;
+    bool valid;
+};
+
+// Map this workgroup to its logical tile (XCD-aware, see file header).
+__device__ __forceinline__ TileCoord locate_tile(const TileTable *table) {
+    TileCoord tc;
+    tc.valid = false;
+    const int total = table->total_tiles;
+    const int per_xcd = (total + 7) >> 3;
+    const int xcd = blockIdx.x & 7;
+    const int slot = blockIdx.x >> 3;
+    if (slot >= per_xcd) return tc;
+    const int logical = xcd * per_xcd + slot;
+    if (logical >= total) return tc;
+    int lo = 0, hi = table->num_entries;  // last entry with tile_begin <= logical
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (table->entries[mid].tile_begin <= logical) lo = mid; else hi = mid;
+    }
+    tc.e = table->entries[lo];
+    const int r = logical - tc.e.tile_begin;
+    tc.col_tile = r / tc.e.num_row_tiles;
+    tc.row_tile = r - tc.col_tile * tc.e.num_row_tiles;
+    tc.valid = true;
+    return tc;
+}
+
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int kTileBytes = BM * BK * 2;                 // 32 KB per operand per stage
+constexpr int kLdsBytes16 = 4 * kTileBytes;             // A,B x 2 stages = 128 KB
+
+enum OutMode { OUT_SAME = 0, OUT_F32 = 1, ACC_F32 = 2 };
+
+template <int DT>
+__device__ __forceinline__ f32x16 mfma16(v16 a, v16 b, f32x16 c) {
+    if constexpr (DT == MS_BF16) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                       0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                      0, 0);
+    }
+}
+
+// LDS swizzle: 16-byte chunk position of (row, chunk) inside the row's 128 bytes.
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+
+// Fast 16-bit kernels (gmm_fast.hip).  Returns MS_OK after launching, or -1 if
+// this problem does not meet the fast kernels' alignment conditions.
+int launch_gmm16_fast(hipStream_t stream, const GmmArgs &args, int dtype, int out_mode, bool a_red, bool b_red,
+                      unsigned grid);
+
+}  // namespace ms
