@@ -1,20 +1,29 @@
-// Fast path of the 16-bit grouped matmul for gfx950: same 256x256x64 macro tile and
-// LDS layout as the generic kernel, but for problems whose pointers and strides
-// allow 16-byte vector access everywhere.  All edge handling is branch-free
-// (clamped addresses, zero masks on the reduction tail), global loads use a
-// uniform 64-bit tile base plus per-lane 32-bit offsets, and the K loop is
-// software-pipelined by hand so that global loads are in flight all the time:
+// Fast path of the 16-bit grouped matmul for gfx950: 256x256x64 macro tile per
+// 256-thread workgroup (2x2 wavefronts, 128x128 per wavefront = 4x4
+// v_mfma_f32_32x32x16), for problems whose pointers and strides allow 16-byte
+// vector access everywhere.  All edge handling is branch-free (clamped addresses,
+// zero masks on the reduction tail).
 //
+// LDS layout per operand tile
+//   * operand contiguous along the reduction dim in memory ("RED"): stored as
+//     [outer][64 reduction] rows of 128 bytes with an XOR swizzle of the 16-byte
+//     chunks; MFMA fragments are read with ds_read_b128 (bank-conflict free).
+//   * operand contiguous along the outer dim (row of A / column of B): stored as it
+//     lies in memory, [64 reduction][256 outer] with a row pitch of 576 bytes, and the
+//     MFMA fragments (8 consecutive reduction values per lane) are produced by the
+//     transposing LDS read ds_read_b64_tr_b16.  No register transposition, and the
+//     global loads stay fully coalesced (32 lanes x 16 bytes per memory row).
+//
+// K loop, software-pipelined by hand so that global loads are in flight all the time:
 //   registers hold tile kt+1 (loaded one K step ago), LDS stage `cur` holds tile kt.
 //   step kt, phase p = 0..3 (one 16-wide slice of the 64-wide K step each):
 //       store part p of tile kt+1 from registers to LDS stage `nxt`
 //       issue the global loads of part p of tile kt+2 into the same registers
 //       read the MFMA fragments of slice p+1 from LDS stage `cur`
 //       16 MFMAs on the fragments of slice p
-//   (parts: A rows/ks 0-3, A 4-7, B 0-3, B 4-7 of each lane's eight 16-byte loads)
+//   (parts: loads 0-3 / 4-7 of A, loads 0-3 / 4-7 of B, of each lane's eight per operand)
 //   in phase 3 a workgroup barrier sits between the two halves of the MFMAs; after it
 //   the fragments of slice 0 of tile kt+1 are read from stage `nxt`.
-//
 // Every load therefore has a full K step (64 MFMAs per wavefront) to arrive, and the
 // vector memory path sees a steady request stream instead of one burst per step.
 #include <type_traits>
@@ -29,22 +38,39 @@ constexpr int SG_MFMA = 0x008, SG_VMEM_RD = 0x020, SG_DS_RD = 0x100, SG_DS_WR = 
 
 template <int MASK, int N, int ID>
 __device__ __forceinline__ void sg() {
-    __builtin_amdgcn_sched_group_barrier(MASK, N, ID);
+    if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, ID);
 }
 
-// Per-lane global offsets (bytes, relative to the tile's uniform base pointer) of the
-// 8 sixteen-byte loads this lane issues per K step.
+constexpr int kPitchT = 576;                      // row pitch of an outer-contiguous tile: 512 + 64 bytes
+constexpr int kRedTileBytes = 256 * 128;          // [256 outer][64 red] x 2 bytes
+constexpr int kOuterTileBytes = 64 * kPitchT;     // [64 red][256 outer] x 2 bytes, padded rows
+
 template <bool RED>
-struct FastLoader {
-    unsigned off[8];
-    unsigned off0;     // !RED: offset of (reduction index 0, this lane's outer chunk), always valid
-    unsigned lds_off;  // byte offset of this lane's first LDS store inside an operand tile
+constexpr int tile_bytes() { return RED ? kRedTileBytes : kOuterTileBytes; }
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint2 lds_read_tr(const char *p) {
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) s16x4 *)(p));
+    return __builtin_bit_cast(uint2, v);
+}
+
+// One operand of the macro tile: global -> registers -> LDS, and LDS -> MFMA fragments.
+template <bool RED>
+struct Operand {
+    unsigned off[8];    // per-lane global byte offsets of the 8 loads, relative to the tile's base pointer
+    unsigned off0;      // !RED: offset of (reduction index 0, this lane's outer chunk), always valid
+    unsigned st_off;    // byte offset of this lane's first LDS store inside the tile
+    unsigned frag_off;  // byte offset of this lane's fragment reads inside the tile
     v16 r[8];
 
-    // outer0: first outer index of the tile, outer_last: last valid outer index (clamp bound,
-    // for !RED the last valid start of an 8-wide chunk), strides in elements.
-    __device__ __forceinline__ void init(int64_t stride_outer, int64_t stride_red, int outer0, int outer_last) {
+    // outer0: first outer index of the tile; outer_last: clamp bound (RED: last valid outer index,
+    // !RED: last valid start of an 8-wide chunk); wave_outer: this wavefront's first outer index in the tile.
+    __device__ __forceinline__ void init(int64_t stride_outer, int64_t stride_red, int outer0, int outer_last,
+                                         int wave_outer) {
         const int tid = threadIdx.x;
+        const int lane = tid & 63;
         if constexpr (RED) {
             const int ck = tid & 7;
             const int row = tid >> 3;
@@ -55,17 +81,25 @@ struct FastLoader {
                 off[i] = static_cast<unsigned>((static_cast<int64_t>(outer - outer0) * stride_outer + ck * 8) * 2);
             }
             off0 = 0;
-            lds_off = row * 128 + ((ck ^ swz(row)) << 4);
+            st_off = row * 128 + ((ck ^ swz(row)) << 4);
+            const int frow = lane & 31;
+            frag_off = (wave_outer + frow) * 128 + (((lane >> 5) ^ swz(frow)) << 4);
         } else {
-            const int kb = tid & 7;
-            const int nb = tid >> 3;
-            int outer = outer0 + nb * 8;
+            const int chunk = tid & 31;   // 16-byte chunk along the outer dim
+            const int rrow = tid >> 5;    // reduction row within a group of 8
+            int outer = outer0 + chunk * 8;
             outer = outer > outer_last ? outer_last : outer;
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
-                off[j] = static_cast<unsigned>((static_cast<int64_t>(kb * 8 + j) * stride_red + (outer - outer0)) * 2);
+            for (int i = 0; i < 8; ++i)
+                off[i] = static_cast<unsigned>((static_cast<int64_t>(i * 8 + rrow) * stride_red + (outer - outer0)) * 2);
             off0 = static_cast<unsigned>((outer - outer0) * 2);
-            lds_off = 0;
+            st_off = rrow * kPitchT + chunk * 16;
+            // transposing read: in each group of 16 lanes, lane L supplies the 4-element segment at
+            // (reduction L/4, outer 4*(L%4)) and receives reduction 0..3 of outer L.
+            const int l16 = lane & 15;
+            const int red = 8 * (lane >> 5) + (l16 >> 2);
+            const int out = wave_outer + 16 * ((lane >> 4) & 1) + 4 * (l16 & 3);
+            frag_off = red * kPitchT + out * 2;
         }
     }
 
@@ -79,11 +113,11 @@ struct FastLoader {
             if constexpr (!TAIL) {
                 r[i] = *reinterpret_cast<const v16 *>(base + off[i]);
             } else {
-                // RED: one chunk of 8 reduction indices per lane (whole or nothing: the reduction
-                // extent is a multiple of 8 on this path); !RED: one reduction index per load.
-                // Masked-out lanes read a valid address (chunk 0 / reduction index 0) instead.
+                // RED: one chunk of 8 reduction indices per lane (whole or nothing: the reduction extent is a
+                // multiple of 8 on this path); !RED: one reduction index per load.  Masked-out lanes read a
+                // valid address (chunk 0 / reduction index 0) instead.
                 const int q = tid & 7;
-                const bool ok = RED ? (q * 8 < nvalid) : (q * 8 + i < nvalid);
+                const bool ok = RED ? (q * 8 < nvalid) : (i * 8 + (tid >> 5) < nvalid);
                 const unsigned o = ok ? off[i] : (RED ? off[i] - q * 16 : off0);
                 const v16 v = *reinterpret_cast<const v16 *>(base + o);
                 const v16 z = {0u, 0u, 0u, 0u};
@@ -92,25 +126,24 @@ struct FastLoader {
         }
     }
 
-    __device__ __forceinline__ void store_half(char *lds_tile, int h) const {
+    __device__ __forceinline__ void store_half(char *tile, int h) const {
+#pragma unroll
+        for (int i = 4 * h; i < 4 * h + 4; ++i) {
+            if constexpr (RED) *reinterpret_cast<v16 *>(tile + st_off + i * 32 * 128) = r[i];
+            else *reinterpret_cast<v16 *>(tile + st_off + i * 8 * kPitchT) = r[i];
+        }
+    }
+
+    // Fragment t (32 outer indices) of K slice kk (16 reduction indices): 8 consecutive reduction values
+    // of outer index (lane & 31), reduction half (lane >> 5).
+    __device__ __forceinline__ v16 frag(const char *tile, int kk, int t) const {
         if constexpr (RED) {
-#pragma unroll
-            for (int i = 4 * h; i < 4 * h + 4; ++i) *reinterpret_cast<v16 *>(lds_tile + lds_off + i * 32 * 128) = r[i];
+            return *reinterpret_cast<const v16 *>(tile + (frag_off ^ ((kk * 2) << 4)) + t * 32 * 128);
         } else {
-            // 4 (reduction) x 8 (outer) block -> for each outer index 4 reduction values = 8 bytes
-            const int tid = threadIdx.x;
-            const int kb = tid & 7;
-            const int nb = tid >> 3;
-#pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                uint2 o;
-                // bytes of {hi:lo}: low halves -> 0x05040100, high halves -> 0x07060302
-                const unsigned sel = (c & 1) ? 0x07060302u : 0x05040100u;
-                o.x = __builtin_amdgcn_perm(r[4 * h + 1][c >> 1], r[4 * h][c >> 1], sel);
-                o.y = __builtin_amdgcn_perm(r[4 * h + 3][c >> 1], r[4 * h + 2][c >> 1], sel);
-                const int row = nb * 8 + c;
-                *reinterpret_cast<uint2 *>(lds_tile + row * 128 + ((kb ^ swz(row)) << 4) + h * 8) = o;
-            }
+            const char *p = tile + frag_off + kk * 16 * kPitchT + t * 64;
+            const uint2 lo = lds_read_tr(p);
+            const uint2 hi = lds_read_tr(p + 4 * kPitchT);
+            return v16{lo.x, lo.y, hi.x, hi.y};
         }
     }
 };
@@ -118,6 +151,8 @@ struct FastLoader {
 template <int DT, bool A_RED, bool B_RED, int OUT>
 __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
+    constexpr int A_BYTES = tile_bytes<A_RED>();
+    constexpr int STAGE = A_BYTES + tile_bytes<B_RED>();
     const TileCoord tc = locate_tile(p.table);
     if (!tc.valid) return;
 
@@ -125,6 +160,7 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
+    const int hi = lane >> 5;
 
     const int row0 = tc.e.row_begin + tc.row_tile * BM;
     const int row_end = tc.e.row_end;
@@ -140,17 +176,10 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    // per-lane fragment read offsets (bytes) inside an operand tile
-    const int frow = lane & 31;
-    const int hi = lane >> 5;
-    const int fbase = frow * 128 + ((hi ^ swz(frow)) << 4);   // chunk (kk*2+hi)^swz = (kk*2) ^ (hi^swz)
-    const int a_frag = wm * 128 * 128 + fbase;
-    const int b_frag = wn * 128 * 128 + fbase;
-
-    FastLoader<A_RED> la;
-    FastLoader<B_RED> lb;
-    la.init(p.a_stride_row, p.a_stride_red, row0, A_RED ? row_end - 1 : row_end - 8);
-    lb.init(p.b_stride_col, p.b_stride_red, col0, B_RED ? col_end - 1 : col_end - 8);
+    Operand<A_RED> la;
+    Operand<B_RED> lb;
+    la.init(p.a_stride_row, p.a_stride_red, row0, A_RED ? row_end - 1 : row_end - 8, wm * 128);
+    lb.init(p.b_stride_col, p.b_stride_red, col0, B_RED ? col_end - 1 : col_end - 8, wn * 128);
     // uniform base pointers of element (outer0, red_begin); advanced by one K step per iteration
     const char *a_ptr = static_cast<const char *>(p.a) +
                         (static_cast<int64_t>(row0) * p.a_stride_row + static_cast<int64_t>(red_begin) * p.a_stride_red) * 2;
@@ -165,11 +194,10 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
 
     v16 af[2][4], bf[2][4];
     auto read_frags = [&](const char *stage, int set, int kk) {
-        const int koff = (kk * 2) << 4;   // XOR term of the fragment's chunk
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            af[set][t] = *reinterpret_cast<const v16 *>(stage + (a_frag ^ koff) + t * 32 * 128);
-            bf[set][t] = *reinterpret_cast<const v16 *>(stage + kTileBytes + (b_frag ^ koff) + t * 32 * 128);
+            af[set][t] = la.frag(stage, kk, t);
+            bf[set][t] = lb.frag(stage + A_BYTES, kk, t);
         }
     };
     auto mfmas = [&](int set, int i0, int i1) {
@@ -179,14 +207,14 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
             for (int j = 0; j < 4; ++j) acc[i][j] = mfma16<DT>(bf[set][j], af[set][i], acc[i][j]);
     };
     // part p of a tile: p = 0,1 -> A halves, p = 2,3 -> B halves
-    auto load_part = [&](auto tail_c, int p, int nvalid) {
+    auto load_part = [&](auto tail_c, int part, int nvalid) {
         constexpr bool TAIL = decltype(tail_c)::value;
-        if (p < 2) la.template load_half<TAIL>(a_ptr, nvalid, p);
-        else lb.template load_half<TAIL>(b_ptr, nvalid, p - 2);
+        if (part < 2) la.template load_half<TAIL>(a_ptr, nvalid, part);
+        else lb.template load_half<TAIL>(b_ptr, nvalid, part - 2);
     };
-    auto store_part = [&](char *stage, int p) {
-        if (p < 2) la.store_half(stage, p);
-        else lb.store_half(stage + kTileBytes, p - 2);
+    auto store_part = [&](char *stage, int part) {
+        if (part < 2) la.store_half(stage, part);
+        else lb.store_half(stage + A_BYTES, part - 2);
     };
     auto lds_barrier = [&]() {
         __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0) only: global loads stay in flight
@@ -198,26 +226,29 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
         // consumed at once), so no load is outstanding when the steady-state loop is entered and the
         // loop's own issue order alone decides how long each of its waits has to be.
 #pragma unroll
-        for (int p = 0; p < 4; ++p) load_part(std::true_type{}, p, red_len);
+        for (int part = 0; part < 4; ++part) load_part(std::true_type{}, part, red_len);
 #pragma unroll
-        for (int p = 0; p < 4; ++p) store_part(lds, p);
+        for (int part = 0; part < 4; ++part) store_part(lds, part);
         if (nk > 1) {
             a_ptr += a_step;
             b_ptr += b_step;
 #pragma unroll
-            for (int p = 0; p < 4; ++p) load_part(std::true_type{}, p, red_len - BK);
+            for (int part = 0; part < 4; ++part) load_part(std::true_type{}, part, red_len - BK);
         }
         lds_barrier();
         read_frags(lds, 0, 0);
     }
 
+    // LDS fragment-read instructions per 16-MFMA phase (ds_read_b128 x4 or ds_read_b64_tr x8 per operand)
+    constexpr int NRD = (A_RED ? 4 : 8) + (B_RED ? 4 : 8);
+
     int kt = 0;
-    // HAS1: tile kt+1 exists (it is in registers); HAS2: tile kt+2 exists; TAIL2: tile kt+2 is the last one.
+    // HAS1: tile kt+1 exists (it is in registers); HAS2: tile kt+2 exists; tail2_c: tile kt+2 is the last one.
     auto k_step = [&](auto has1_c, auto has2_c, auto tail2_c) {
         constexpr bool HAS1 = decltype(has1_c)::value;
         constexpr bool HAS2 = decltype(has2_c)::value;
-        const char *cur = lds + (kt & 1) * 2 * kTileBytes;
-        char *nxt = lds + ((kt + 1) & 1) * 2 * kTileBytes;
+        const char *cur = lds + (kt & 1) * STAGE;
+        char *nxt = lds + ((kt + 1) & 1) * STAGE;
         if constexpr (HAS2) {
             a_ptr += a_step;
             b_ptr += b_step;
@@ -235,21 +266,19 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
                 for (int g = 0; g < 8; ++g) {
                     sg<SG_DS_RD, 1, 0>();
                     sg<SG_MFMA, 1, 0>();
-                    if (HAS1 && g < 4) sg<SG_DS_WR, (A_RED && B_RED) ? 1 : 2, 0>();
-                    if (HAS2 && g >= 4) sg<SG_VMEM_RD, 1, 0>();
+                    if (g < 4) sg<SG_DS_WR, HAS1 ? 1 : 0, 0>(); else sg<SG_VMEM_RD, HAS2 ? 1 : 0, 0>();
+                    if (NRD == 16 || (NRD == 12 && (g & 1))) sg<SG_DS_RD, 1, 0>();
                     sg<SG_MFMA, 1, 0>();
                 }
                 __builtin_amdgcn_sched_barrier(0);
             } else {
                 mfmas(set, 0, 2);
-                if constexpr (HAS1) {
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        sg<SG_DS_WR, (A_RED && B_RED) ? 1 : 2, 0>();
-                        sg<SG_MFMA, 1, 0>();
-                        if (HAS2) sg<SG_VMEM_RD, 1, 0>();
-                        sg<SG_MFMA, 1, 0>();
-                    }
+                for (int g = 0; g < 4; ++g) {
+                    sg<SG_DS_WR, HAS1 ? 1 : 0, 0>();
+                    sg<SG_MFMA, 1, 0>();
+                    sg<SG_VMEM_RD, HAS2 ? 1 : 0, 0>();
+                    sg<SG_MFMA, 1, 0>();
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr (HAS1) {
@@ -260,7 +289,8 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
                 if constexpr (HAS1) {
 #pragma unroll
                     for (int g = 0; g < 8; ++g) {
-                        sg<SG_DS_RD, 1, 1>();
+                        sg<SG_DS_RD, NRD / 8, 1>();
+                        if (NRD == 12 && (g & 1)) sg<SG_DS_RD, 1, 1>();
                         sg<SG_MFMA, 1, 1>();
                     }
                 }
@@ -314,11 +344,12 @@ int launch_fast(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red,
     else if (a_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, false, OUT>);
     else if (b_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, true, OUT>);
     else fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, false, OUT>);
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes16);
+    const int lds_bytes = 2 * ((a_red ? kRedTileBytes : kOuterTileBytes) + (b_red ? kRedTileBytes : kOuterTileBytes));
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "ms_gmm: hipFuncSetAttribute: %s", hipGetErrorString(e));
     GmmArgs copy = args;
     void *kargs[] = {&copy};
-    e = hipLaunchKernel(fn, dim3(grid), dim3(256), kargs, kLdsBytes16, stream);
+    e = hipLaunchKernel(fn, dim3(grid), dim3(256), kargs, lds_bytes, stream);
     MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "ms_gmm: launch failed: %s", hipGetErrorString(e));
     return MS_OK;
 }
