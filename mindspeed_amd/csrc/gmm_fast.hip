@@ -48,6 +48,10 @@ constexpr int kOuterTileBytes = 64 * kPitchT;     // [64 red][256 outer] x 2 byt
 template <bool RED>
 constexpr int tile_bytes() { return RED ? kRedTileBytes : kOuterTileBytes; }
 
+constexpr int kStagePitch = 264;                          // epilogue staging: 128 x 2 bytes + 8 bytes pad
+constexpr int kStagePerWave = 128 * kStagePitch;          // one 128 x 128 16-bit block per wavefront
+constexpr int kStageBytes = 4 * kStagePerWave;
+
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint2 lds_read_tr(const char *p) {
@@ -306,29 +310,54 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
     // Epilogue.  acc[i][j][4*q+e] = C[row0 + wm*128 + i*32 + (lane&31)]
     //                                [col0 + wn*128 + j*32 + 8*q + 4*(lane>>5) + e]
     const int64_t ldc = p.c_stride_row;
-    const bool full_cols = col0 + BN <= col_end;
+    if constexpr (OUT == OUT_SAME) {
+        // 16-bit output: each wavefront stages its 128x128 block in its own LDS region (row pitch 264
+        // bytes: conflict-free for the 8-byte column-slice writes and the row reads) and writes it out
+        // as 16 bytes per lane, 256 contiguous bytes per row.
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_s_barrier();          // every wavefront is done reading the operand stages
+        char *stg = lds + wave * kStagePerWave;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = row0 + wm * 128 + i * 32 + (lane & 31);
-        if (row >= row_end) continue;
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int col = col0 + wn * 128 + j * 32 + 8 * q + 4 * hi;
-                if (!full_cols && col >= col_end) continue;   // cols is a multiple of 4 on this path
-                const int64_t at = tc.e.c_off + static_cast<int64_t>(row) * ldc + col;
-                float v[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
-                if constexpr (OUT == OUT_SAME) {
+                for (int q = 0; q < 4; ++q) {
                     uint16_t h[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) h[e] = DT == MS_BF16 ? BF16::from_float(v[e]) : FP16::from_float(v[e]);
-                    *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(p.c) + at) = *reinterpret_cast<uint2 *>(h);
-                } else {
-                    float *c = static_cast<float *>(p.c) + at;
-                    f32x4 o = {v[0], v[1], v[2], v[3]};
+                    for (int e = 0; e < 4; ++e)
+                        h[e] = DT == MS_BF16 ? BF16::from_float(acc[i][j][4 * q + e]) : FP16::from_float(acc[i][j][4 * q + e]);
+                    *reinterpret_cast<uint2 *>(stg + (i * 32 + (lane & 31)) * kStagePitch + (j * 32 + 8 * q + 4 * hi) * 2) =
+                        *reinterpret_cast<uint2 *>(h);
+                }
+        __builtin_amdgcn_s_waitcnt(0xC07F);    // own writes only: the region is private to this wavefront
+        const int chunk = lane & 15;           // 8 columns = 16 bytes
+        const int col = col0 + wn * 128 + chunk * 8;
+        const bool col_ok = col < col_end;     // cols is a multiple of 8 on this path
+        uint16_t *cbase = static_cast<uint16_t *>(p.c) + tc.e.c_off + col;
+#pragma unroll 4
+        for (int pass = 0; pass < 32; ++pass) {
+            const int r = pass * 4 + (lane >> 4);
+            const int row = row0 + wm * 128 + r;
+            const uint2 lo = *reinterpret_cast<const uint2 *>(stg + r * kStagePitch + chunk * 16);
+            const uint2 hi2 = *reinterpret_cast<const uint2 *>(stg + r * kStagePitch + chunk * 16 + 8);
+            if (col_ok && row < row_end)
+                *reinterpret_cast<v16 *>(cbase + static_cast<int64_t>(row) * ldc) = v16{lo.x, lo.y, hi2.x, hi2.y};
+        }
+    } else {
+        const bool full_cols = col0 + BN <= col_end;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = row0 + wm * 128 + i * 32 + (lane & 31);
+            if (row >= row_end) continue;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int col = col0 + wn * 128 + j * 32 + 8 * q + 4 * hi;
+                    if (!full_cols && col >= col_end) continue;   // cols is a multiple of 4 on this path
+                    float *c = static_cast<float *>(p.c) + tc.e.c_off + static_cast<int64_t>(row) * ldc + col;
+                    f32x4 o = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
                     if constexpr (OUT == ACC_F32) o += *reinterpret_cast<f32x4 *>(c);
                     *reinterpret_cast<f32x4 *>(c) = o;
                 }
@@ -344,7 +373,8 @@ int launch_fast(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red,
     else if (a_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, false, OUT>);
     else if (b_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, true, OUT>);
     else fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, false, OUT>);
-    const int lds_bytes = 2 * ((a_red ? kRedTileBytes : kOuterTileBytes) + (b_red ? kRedTileBytes : kOuterTileBytes));
+    int lds_bytes = 2 * ((a_red ? kRedTileBytes : kOuterTileBytes) + (b_red ? kRedTileBytes : kOuterTileBytes));
+    if (OUT == OUT_SAME && lds_bytes < kStageBytes) lds_bytes = kStageBytes;
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "ms_gmm: hipFuncSetAttribute: %s", hipGetErrorString(e));
     GmmArgs copy = args;
