@@ -24,8 +24,8 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const typename DT::storage 
         const S *xu = xg + ffn;
         S g[VEC], u[VEC], o[VEC];
         if constexpr (VEC * sizeof(S) == 16) {
-            *reinterpret_cast<v16 *>(g) = __builtin_nontemporal_load(reinterpret_cast<const v16 *>(xg));
-            *reinterpret_cast<v16 *>(u) = __builtin_nontemporal_load(reinterpret_cast<const v16 *>(xu));
+            *reinterpret_cast<v16 *>(g) = MS_NT_LOAD(reinterpret_cast<const v16 *>(xg));
+            *reinterpret_cast<v16 *>(u) = MS_NT_LOAD(reinterpret_cast<const v16 *>(xu));
         } else {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) { g[e] = xg[e]; u[e] = xu[e]; }
@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const typename DT::storage 
         }
         S *dst = y + r * ffn + c;
         if constexpr (VEC * sizeof(S) == 16) {
-            __builtin_nontemporal_store(*reinterpret_cast<v16 *>(o), reinterpret_cast<v16 *>(dst));
+            MS_NT_STORE(*reinterpret_cast<v16 *>(o), reinterpret_cast<v16 *>(dst));
         } else {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) dst[e] = o[e];
@@ -66,9 +66,9 @@ __global__ __launch_bounds__(256) void swiglu_grad_kernel(const typename DT::sto
         const S *gp = gy + r * ffn + c;
         S g[VEC], u[VEC], d[VEC], og[VEC], ou[VEC];
         if constexpr (VEC * sizeof(S) == 16) {
-            *reinterpret_cast<v16 *>(g) = __builtin_nontemporal_load(reinterpret_cast<const v16 *>(xg));
-            *reinterpret_cast<v16 *>(u) = __builtin_nontemporal_load(reinterpret_cast<const v16 *>(xu));
-            *reinterpret_cast<v16 *>(d) = __builtin_nontemporal_load(reinterpret_cast<const v16 *>(gp));
+            *reinterpret_cast<v16 *>(g) = MS_NT_LOAD(reinterpret_cast<const v16 *>(xg));
+            *reinterpret_cast<v16 *>(u) = MS_NT_LOAD(reinterpret_cast<const v16 *>(xu));
+            *reinterpret_cast<v16 *>(d) = MS_NT_LOAD(reinterpret_cast<const v16 *>(gp));
         } else {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) { g[e] = xg[e]; u[e] = xu[e]; d[e] = gp[e]; }
@@ -86,8 +86,8 @@ __global__ __launch_bounds__(256) void swiglu_grad_kernel(const typename DT::sto
         S *dg = gx + r * 2 * ffn + c;
         S *du = dg + ffn;
         if constexpr (VEC * sizeof(S) == 16) {
-            __builtin_nontemporal_store(*reinterpret_cast<v16 *>(og), reinterpret_cast<v16 *>(dg));
-            __builtin_nontemporal_store(*reinterpret_cast<v16 *>(ou), reinterpret_cast<v16 *>(du));
+            MS_NT_STORE(*reinterpret_cast<v16 *>(og), reinterpret_cast<v16 *>(dg));
+            MS_NT_STORE(*reinterpret_cast<v16 *>(ou), reinterpret_cast<v16 *>(du));
         } else {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) { dg[e] = og[e]; du[e] = ou[e]; }
@@ -145,10 +145,11 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const VecT *__restrict
     const int r = blockIdx.x * (256 / lanes) + local_row;
     if (r >= rows) return;
     const int m = row_map[r];
+    if (static_cast<unsigned>(m) >= static_cast<unsigned>(rows)) return;   // corrupt map entry: touch nothing
     const int64_t s = inverse ? r : m;
     const int64_t d = inverse ? m : r;
     for (int c = lane; c < vecs_per_row; c += lanes)
-        __builtin_nontemporal_store(__builtin_nontemporal_load(in + s * vecs_per_row + c), out + d * vecs_per_row + c);
+        MS_NT_STORE(MS_NT_LOAD(in + s * vecs_per_row + c), out + d * vecs_per_row + c);
 }
 
 template <typename VecT>

@@ -261,8 +261,12 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
             const int set = kk & 1;
+#ifndef EXP_NOSTORE
             if constexpr (HAS1) store_part(nxt, kk);
+#endif
+#ifndef EXP_NOLOAD
             if constexpr (HAS2) load_part(tail2_c, kk, left2);
+#endif
             if (kk < 3) {
                 read_frags(cur, set ^ 1, kk + 1);
                 mfmas(set, 0, 4);

@@ -16,7 +16,7 @@ namespace ms {
 namespace {
 
 constexpr int kSortBlockWaves = 16;          // single-block sort: 1024 threads
-constexpr int kSmallSortMax = 16384;         // flat positions handled by one block
+constexpr int kSmallSortMax = 16384;         // flat positions handled by one block (16 waves x 1024 keys)
 constexpr int kHistWavesPerBlock = 4;        // multi-block sort: 256 threads
 constexpr int kMaxSegments = 4096;
 
@@ -40,42 +40,165 @@ __device__ __forceinline__ unsigned long long match_key(int key, bool valid, int
     return m;
 }
 
-// Histogram of idx[begin, end) into one table row owned by this wavefront.
+constexpr int kKeysPerLane = 16;               // one register-resident chunk: 64 lanes x 16 keys
+constexpr int kChunk = 64 * kKeysPerLane;
+
+// Load up to kChunk keys of idx[begin, end) into registers (-1 past the end).  All loads are issued
+// before any is used, so a chunk costs one memory latency instead of one per 64 keys.
 template <typename IdxT>
-__device__ __forceinline__ void wave_histogram(volatile int *row, const IdxT *idx, int begin, int end,
-                                               int nbins, int nbits) {
+__device__ __forceinline__ void load_keys(const IdxT *idx, int begin, int end, int nbins, int (&keys)[kKeysPerLane]) {
     const int lane = threadIdx.x & 63;
-    for (int base = begin; base < end; base += 64) {
-        const int i = base + lane;
-        const bool valid = i < end;
-        const int key = valid ? load_key(idx, i, nbins) : 0;
-        const unsigned long long m = match_key(key, valid, nbits);
-        if (valid && lane == __ffsll(static_cast<long long>(m)) - 1) row[key] += __popcll(m);
+    if (begin >= end) {
+#pragma unroll
+        for (int u = 0; u < kKeysPerLane; ++u) keys[u] = -1;
+        return;
+    }
+    // Unconditional loads from clamped positions (no per-load branch, so nothing waits in between),
+    // then mask what lies past the end.
+    IdxT raw[kKeysPerLane];
+#pragma unroll
+    for (int u = 0; u < kKeysPerLane; ++u) raw[u] = idx[min(begin + u * 64 + lane, end - 1)];
+#pragma unroll
+    for (int u = 0; u < kKeysPerLane; ++u) {
+        long long v = static_cast<long long>(raw[u]);
+        v = v < 0 ? 0 : v;
+        v = v >= nbins ? nbins - 1 : v;
+        keys[u] = begin + u * 64 + lane < end ? static_cast<int>(v) : -1;
     }
 }
 
-// Stable scatter of idx[begin, end): row[key] holds the next output row of `key`
-// for this wavefront's segment.
-template <typename IdxT>
-__device__ __forceinline__ void wave_scatter(volatile int *row, const IdxT *idx, int begin, int end,
-                                             int nbins, int nbits, int num_out, int32_t *row_id_map,
-                                             int32_t *sorted_indices) {
+// Histogram of a register-resident chunk into one table row owned by this wavefront.  One lane per
+// distinct key (the lowest lane holding it) adds the key's multiplicity with a fire-and-forget LDS add.
+__device__ __forceinline__ void hist_keys(int *row, const int (&keys)[kKeysPerLane], int count, int nbits) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int u = 0; u < kKeysPerLane; ++u) {
+        if (u * 64 >= count) break;
+        const bool valid = keys[u] >= 0;
+        const int key = valid ? keys[u] : 0;
+        const unsigned long long m = match_key(key, valid, nbits);
+        if (valid && lane == __ffsll(static_cast<long long>(m)) - 1) atomicAdd(&row[key], __popcll(m));
+    }
+}
+
+// Stable scatter of a register-resident chunk that starts at flat position `begin`: row[key] holds
+// the next output row of `key` for this wavefront's segment.  The lowest lane of every key fetches
+// and advances that counter with one returning LDS add and hands the old value to the key's lanes.
+__device__ __forceinline__ void scatter_keys(int *row, const int (&keys)[kKeysPerLane], int begin, int count,
+                                             int nbits, int num_out, int32_t *row_id_map, int32_t *sorted_indices) {
     const int lane = threadIdx.x & 63;
     const unsigned long long lt = (1ull << lane) - 1ull;
-    for (int base = begin; base < end; base += 64) {
-        const int i = base + lane;
-        const bool valid = i < end;
-        const int key = valid ? load_key(idx, i, nbins) : 0;
+#pragma unroll
+    for (int u = 0; u < kKeysPerLane; ++u) {
+        if (u * 64 >= count) break;
+        const bool valid = keys[u] >= 0;
+        const int key = valid ? keys[u] : 0;
         const unsigned long long m = match_key(key, valid, nbits);
-        const int first = valid ? row[key] : 0;
-        const int rank = first + __popcll(m & lt);
-        __builtin_amdgcn_wave_barrier();
-        if (valid && lane == __ffsll(static_cast<long long>(m)) - 1) row[key] = first + __popcll(m);
-        __builtin_amdgcn_wave_barrier();
+        const int leader = valid ? __ffsll(static_cast<long long>(m)) - 1 : lane;
+        int first = 0;
+        if (valid && lane == leader) first = atomicAdd(&row[key], __popcll(m));
+        first = __shfl(first, leader, 64);
         if (valid) {
+            const int rank = first + __popcll(m & lt);
+            const int i = begin + u * 64 + lane;
             row_id_map[i] = rank;
             if (sorted_indices != nullptr && rank < num_out) sorted_indices[rank] = i;
         }
+    }
+}
+
+// ---- few bins (<= NB): one ballot per bin, counters in scalar registers ---------------------------
+// With at most 16 bins a ballot per bin is cheaper than matching lanes pairwise: the per-bin counts and
+// running offsets are wave-uniform (scalar registers), and a lane's rank inside the chunk is the number
+// of lower lanes in its bin's ballot.
+__device__ __forceinline__ int lanes_below(unsigned long long mask) {
+    return __builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(mask >> 32),
+                                     __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(mask), 0u));
+}
+
+template <int NB>
+__device__ __forceinline__ void hist_keys_few(int *row, const int (&keys)[kKeysPerLane], int count, int nbins) {
+    const int lane = threadIdx.x & 63;
+    int cnt[NB];
+#pragma unroll
+    for (int e = 0; e < NB; ++e) cnt[e] = 0;
+#pragma unroll
+    for (int u = 0; u < kKeysPerLane; ++u) {
+        if (u * 64 >= count) break;
+#pragma unroll
+        for (int e = 0; e < NB; ++e) cnt[e] += __popcll(__ballot(keys[u] == e));
+    }
+    int mine = 0;
+#pragma unroll
+    for (int e = 0; e < NB; ++e) mine = lane == e ? cnt[e] : mine;
+    if (lane < nbins) row[lane] += mine;   // the row has nbins (<= NB) entries
+}
+
+template <int NB>
+__device__ __forceinline__ void scatter_keys_few(int *row, const int (&keys)[kKeysPerLane], int begin, int count,
+                                                 int nbins, int num_out, int32_t *row_id_map, int32_t *sorted_indices) {
+    const int lane = threadIdx.x & 63;
+    int base[NB];
+    const int mine = lane < nbins ? row[lane] : 0;
+#pragma unroll
+    for (int e = 0; e < NB; ++e) base[e] = __builtin_amdgcn_readlane(mine, e);
+#pragma unroll
+    for (int u = 0; u < kKeysPerLane; ++u) {
+        if (u * 64 >= count) break;
+        int rank = 0;
+#pragma unroll
+        for (int e = 0; e < NB; ++e) {
+            const unsigned long long bal = __ballot(keys[u] == e);
+            rank = keys[u] == e ? base[e] + lanes_below(bal) : rank;
+            base[e] += __popcll(bal);
+        }
+        if (keys[u] >= 0) {
+            const int i = begin + u * 64 + lane;
+            row_id_map[i] = rank;
+            if (sorted_indices != nullptr && rank < num_out) sorted_indices[rank] = i;
+        }
+    }
+    int upd = 0;
+#pragma unroll
+    for (int e = 0; e < NB; ++e) upd = lane == e ? base[e] : upd;
+    if (lane < nbins) row[lane] = upd;
+}
+
+// Dispatch on the bin count.
+__device__ __forceinline__ void hist_chunk(int *row, const int (&keys)[kKeysPerLane], int count, int nbins, int nbits) {
+    if (nbins <= 8) hist_keys_few<8>(row, keys, count, nbins);
+    else if (nbins <= 16) hist_keys_few<16>(row, keys, count, nbins);
+    else hist_keys(row, keys, count, nbits);
+}
+__device__ __forceinline__ void scatter_chunk(int *row, const int (&keys)[kKeysPerLane], int begin, int count, int nbins,
+                                              int nbits, int num_out, int32_t *row_id_map, int32_t *sorted_indices) {
+    if (nbins <= 8) scatter_keys_few<8>(row, keys, begin, count, nbins, num_out, row_id_map, sorted_indices);
+    else if (nbins <= 16) scatter_keys_few<16>(row, keys, begin, count, nbins, num_out, row_id_map, sorted_indices);
+    else scatter_keys(row, keys, begin, count, nbits, num_out, row_id_map, sorted_indices);
+}
+
+// Histogram of idx[begin, end) into one table row owned by this wavefront.
+template <typename IdxT>
+__device__ __forceinline__ void wave_histogram(int *row, const IdxT *idx, int begin, int end,
+                                               int nbins, int nbits) {
+    int keys[kKeysPerLane];
+    for (int c = begin; c < end; c += kChunk) {
+        const int ce = min(c + kChunk, end);
+        load_keys(idx, c, ce, nbins, keys);
+        hist_chunk(row, keys, ce - c, nbins, nbits);
+    }
+}
+
+// Stable scatter of idx[begin, end).
+template <typename IdxT>
+__device__ __forceinline__ void wave_scatter(int *row, const IdxT *idx, int begin, int end,
+                                             int nbins, int nbits, int num_out, int32_t *row_id_map,
+                                             int32_t *sorted_indices) {
+    int keys[kKeysPerLane];
+    for (int c = begin; c < end; c += kChunk) {
+        const int ce = min(c + kChunk, end);
+        load_keys(idx, c, ce, nbins, keys);
+        scatter_chunk(row, keys, c, ce - c, nbins, nbits, num_out, row_id_map, sorted_indices);
     }
 }
 
@@ -121,23 +244,29 @@ __global__ __launch_bounds__(kSortBlockWaves * 64) void sort_small_kernel(
     seg = (seg + 63) & ~63;
     const int begin = min(wave * seg, n);
     const int end = min(begin + seg, n);
-    wave_histogram(lds + wave * nbins, idx, begin, end, nbins, nbits);
+    int keys[kKeysPerLane];                    // seg <= kChunk: the whole segment stays in registers
+    load_keys(idx, begin, end, nbins, keys);
+    hist_chunk(lds + wave * nbins, keys, end - begin, nbins, nbits);
     __syncthreads();
     int total = 0;
+    int cnt[kSortBlockWaves];
     if (tid < nbins) {
-        for (int w = 0; w < kSortBlockWaves; ++w) {
-            const int c = lds[w * nbins + tid];
-            lds[w * nbins + tid] = total;
-            total += c;
-        }
+#pragma unroll
+        for (int w = 0; w < kSortBlockWaves; ++w) cnt[w] = lds[w * nbins + tid];
+#pragma unroll
+        for (int w = 0; w < kSortBlockWaves; ++w) total += cnt[w];
     }
-    const int excl = block_exclusive_scan(total, scratch);
+    int run = block_exclusive_scan(total, scratch);
     if (tid < nbins) {
-        for (int w = 0; w < kSortBlockWaves; ++w) lds[w * nbins + tid] += excl;
+#pragma unroll
+        for (int w = 0; w < kSortBlockWaves; ++w) {
+            lds[w * nbins + tid] = run;
+            run += cnt[w];
+        }
         if (tokens_per_expert != nullptr && tid < tpe_n) tokens_per_expert[tid] = total;
     }
     __syncthreads();
-    wave_scatter(lds + wave * nbins, idx, begin, end, nbins, nbits, num_out, row_id_map, sorted_indices);
+    scatter_chunk(lds + wave * nbins, keys, begin, end - begin, nbins, nbits, num_out, row_id_map, sorted_indices);
 }
 
 // ---- multi-block sort (large inputs): histogram, scan, scatter ----------------------
@@ -166,16 +295,18 @@ __global__ __launch_bounds__(1024) void sort_scan_kernel(int *table, int nseg, i
     const int tid = threadIdx.x;
     int total = 0;
     if (tid < nbins) {
+#pragma unroll 8
+        for (int s = 0; s < nseg; ++s) total += table[static_cast<int64_t>(s) * nbins + tid];
+    }
+    int run = block_exclusive_scan(total, scratch);
+    if (tid < nbins) {
+#pragma unroll 8
         for (int s = 0; s < nseg; ++s) {
             const int64_t at = static_cast<int64_t>(s) * nbins + tid;
             const int c = table[at];
-            table[at] = total;
-            total += c;
+            table[at] = run;
+            run += c;
         }
-    }
-    const int excl = block_exclusive_scan(total, scratch);
-    if (tid < nbins) {
-        for (int s = 0; s < nseg; ++s) table[static_cast<int64_t>(s) * nbins + tid] += excl;
         if (tokens_per_expert != nullptr && tid < tpe_n) tokens_per_expert[tid] = total;
     }
 }
@@ -202,16 +333,19 @@ __global__ __launch_bounds__(kHistWavesPerBlock * 64) void sort_scatter_kernel(
 // rows_per_block rows, `lanes` threads per row, each thread striding over the
 // row's vectors.
 struct RowLayout {
-    int lanes;           // threads per row (power of two, 1..256)
+    int lanes;           // threads per row (power of two, 1..64)
     int rows_per_block;  // 256 / lanes
 };
 inline RowLayout row_layout(int64_t vecs_per_row) {
     int lanes = 1;
-    while (lanes < 256 && lanes < vecs_per_row) lanes <<= 1;
+    while (lanes < 64 && lanes < vecs_per_row) lanes <<= 1;   // one wavefront per row at most
     return RowLayout{lanes, 256 / lanes};
 }
 
-// permuted[row_id_map[t*k+j]] = tokens[t] for every kept (t, j).
+constexpr int kSlotBatch = 8;   // top-k slots whose row ids / weights are kept in registers at a time
+
+// permuted[row_id_map[t*k+j]] = tokens[t] for every kept (t, j).  Row ids are read once per thread,
+// and four independent 16-byte loads are in flight per thread before the first store.
 template <typename VecT>
 __global__ __launch_bounds__(256) void permute_rows_kernel(const VecT *__restrict__ tokens,
                                                            VecT *__restrict__ permuted,
@@ -223,17 +357,32 @@ __global__ __launch_bounds__(256) void permute_rows_kernel(const VecT *__restric
     const int t = blockIdx.x * (256 / lanes) + local_row;
     if (t >= num_tokens) return;
     const VecT *src = tokens + static_cast<int64_t>(t) * vecs_per_row;
-    for (int c = lane; c < vecs_per_row; c += lanes) {
-        const VecT v = __builtin_nontemporal_load(src + c);
-        for (int j = 0; j < topk; ++j) {
-            const int d = row_id_map[static_cast<int64_t>(t) * topk + j];
-            if (d < num_out) __builtin_nontemporal_store(v, permuted + static_cast<int64_t>(d) * vecs_per_row + c);
+    for (int j0 = 0; j0 < topk; j0 += kSlotBatch) {
+        int d[kSlotBatch];
+#pragma unroll
+        for (int j = 0; j < kSlotBatch; ++j)
+            d[j] = j0 + j < topk ? row_id_map[static_cast<int64_t>(t) * topk + j0 + j] : num_out;
+        for (int c0 = lane; c0 < vecs_per_row; c0 += 4 * lanes) {
+            VecT v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
+#pragma unroll
+            for (int j = 0; j < kSlotBatch; ++j) {
+                if (static_cast<unsigned>(d[j]) >= static_cast<unsigned>(num_out)) continue;   // dropped (or corrupt) id
+                VecT *dst = permuted + static_cast<int64_t>(d[j]) * vecs_per_row;
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (c0 + u * lanes < vecs_per_row) dst[c0 + u * lanes] = v[u];
+            }
         }
     }
 }
 
 // out[t] = sum_j w[t,j] * rows[row_id_map[t*k+j]] ; w == nullptr -> unweighted.
 // VEC: elements per thread access (16 bytes worth, or 1 for the unaligned path).
+// Row ids and weights are read once per thread; per pair of output vectors all topk row loads are
+// independent and issued together; accumulation is fp32 in registers, one rounding.
 template <typename DT, int VEC>
 __global__ __launch_bounds__(256) void gather_combine_kernel(
     const typename DT::storage *__restrict__ rows, const int32_t *__restrict__ row_id_map,
@@ -245,34 +394,64 @@ __global__ __launch_bounds__(256) void gather_combine_kernel(
     const int t = blockIdx.x * (256 / lanes) + local_row;
     if (t >= num_tokens) return;
     const int vecs = hidden / VEC;
-    for (int c = lane; c < vecs; c += lanes) {
-        float acc[VEC];
+    constexpr int U = 2;
+    for (int c0 = lane; c0 < vecs; c0 += U * lanes) {
+        float acc[U][VEC];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
-        for (int j = 0; j < topk; ++j) {
-            const int d = row_id_map[static_cast<int64_t>(t) * topk + j];
-            if (d >= num_rows) continue;
-            const float w = probs != nullptr ? DT::to_float(probs[static_cast<int64_t>(t) * topk + j]) : 1.f;
-            const S *src = rows + static_cast<int64_t>(d) * hidden + static_cast<int64_t>(c) * VEC;
-            S tmp[VEC];
-            if constexpr (VEC * sizeof(S) == 16) {
-                *reinterpret_cast<v16 *>(tmp) = __builtin_nontemporal_load(reinterpret_cast<const v16 *>(src));
-            } else {
+        for (int u = 0; u < U; ++u)
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) tmp[e] = src[e];
+            for (int e = 0; e < VEC; ++e) acc[u][e] = 0.f;
+        for (int j0 = 0; j0 < topk; j0 += kSlotBatch) {
+            int d[kSlotBatch];
+            float w[kSlotBatch];
+#pragma unroll
+            for (int j = 0; j < kSlotBatch; ++j) {
+                const int64_t flat = static_cast<int64_t>(t) * topk + j0 + j;
+                d[j] = j0 + j < topk ? row_id_map[flat] : num_rows;
+                w[j] = (probs != nullptr && j0 + j < topk) ? DT::to_float(probs[flat]) : 1.f;
+            }
+            S tmp[kSlotBatch][U][VEC];
+#pragma unroll
+            for (int j = 0; j < kSlotBatch; ++j) {
+                if (static_cast<unsigned>(d[j]) >= static_cast<unsigned>(num_rows)) continue;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int c = c0 + u * lanes;
+                    if (c >= vecs) continue;
+                    const S *src = rows + static_cast<int64_t>(d[j]) * hidden + static_cast<int64_t>(c) * VEC;
+                    if constexpr (VEC * sizeof(S) == 16) {
+                        *reinterpret_cast<v16 *>(tmp[j][u]) = *reinterpret_cast<const v16 *>(src);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) tmp[j][u][e] = src[e];
+                    }
+                }
             }
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) acc[e] = fmaf(w, DT::to_float(tmp[e]), acc[e]);
+            for (int j = 0; j < kSlotBatch; ++j) {
+                if (static_cast<unsigned>(d[j]) >= static_cast<unsigned>(num_rows)) continue;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    if (c0 + u * lanes >= vecs) continue;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc[u][e] = fmaf(w[j], DT::to_float(tmp[j][u][e]), acc[u][e]);
+                }
+            }
         }
-        S res[VEC];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) res[e] = DT::from_float(acc[e]);
-        S *dst = out + static_cast<int64_t>(t) * hidden + static_cast<int64_t>(c) * VEC;
-        if constexpr (VEC * sizeof(S) == 16) {
-            __builtin_nontemporal_store(*reinterpret_cast<v16 *>(res), reinterpret_cast<v16 *>(dst));
-        } else {
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * lanes;
+            if (c >= vecs) continue;
+            S res[VEC];
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) dst[e] = res[e];
+            for (int e = 0; e < VEC; ++e) res[e] = DT::from_float(acc[u][e]);
+            S *dst = out + static_cast<int64_t>(t) * hidden + static_cast<int64_t>(c) * VEC;
+            if constexpr (VEC * sizeof(S) == 16) {
+                *reinterpret_cast<v16 *>(dst) = *reinterpret_cast<v16 *>(res);
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) dst[e] = res[e];
+            }
         }
     }
 }
@@ -292,7 +471,7 @@ __global__ __launch_bounds__(256) void unpermute_grad_kernel(
     for (int j = 0; j < topk; ++j) {
         const int64_t flat = static_cast<int64_t>(t) * topk + j;
         const int d = row_id_map[flat];
-        const bool kept = d < num_rows;
+        const bool kept = static_cast<unsigned>(d) < static_cast<unsigned>(num_rows);   // negative ids count as dropped
         const float w = probs != nullptr ? DT::to_float(probs[flat]) : 1.f;
         float dot = 0.f;
         if (kept) {
@@ -304,7 +483,7 @@ __global__ __launch_bounds__(256) void unpermute_grad_kernel(
                     *reinterpret_cast<v16 *>(g) = *reinterpret_cast<const v16 *>(gp);
                     if (grad_probs != nullptr)
                         *reinterpret_cast<v16 *>(x) =
-                            __builtin_nontemporal_load(reinterpret_cast<const v16 *>(permuted + off));
+                            MS_NT_LOAD(reinterpret_cast<const v16 *>(permuted + off));
                 } else {
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) g[e] = gp[e];
@@ -320,7 +499,7 @@ __global__ __launch_bounds__(256) void unpermute_grad_kernel(
                     if (grad_probs != nullptr) dot = fmaf(gf, DT::to_float(x[e]), dot);
                 }
                 if constexpr (VEC * sizeof(S) == 16) {
-                    __builtin_nontemporal_store(*reinterpret_cast<v16 *>(o),
+                    MS_NT_STORE(*reinterpret_cast<v16 *>(o),
                                                 reinterpret_cast<v16 *>(grad_permuted + off));
                 } else {
 #pragma unroll

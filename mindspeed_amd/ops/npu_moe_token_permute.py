@@ -76,6 +76,7 @@ class _MoeTokenPermute(torch.autograd.Function):
         permuted, row_id_map, sorted_idx, counts, topk = _permute_forward(
             tokens, indices, num_out, num_experts, want_sorted, want_counts)
         ctx.save_for_backward(row_id_map)
+        ctx.set_materialize_grads(False)   # no zero-filled gradients for the integer outputs
         ctx.num_tokens = tokens.size(0)
         ctx.topk = topk
         outs = [permuted, row_id_map]
@@ -91,6 +92,8 @@ class _MoeTokenPermute(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_permuted, *_unused):
         (row_id_map,) = ctx.saved_tensors
+        if grad_permuted is None:
+            return None, None, None, None, None, None
         # npu_moe_token_permute.cpp:53-63,99-118
         if grad_permuted.dim() != 2:
             raise RuntimeError("The dims of input grad_permuted_tokens should be 2 dimensional, "

@@ -45,6 +45,7 @@ class _SortChunks(torch.autograd.Function):
                 _lib.dtype_code(p.dtype, "probs") if p is not None else 0, _lib.ptr(out), _lib.ptr(out_p),
                 _lib.ptr(row_map)), "ms_sort_chunks")
         ctx.save_for_backward(row_map)
+        ctx.set_materialize_grads(False)
         ctx.has_probs = p is not None
         ctx.mark_non_differentiable(row_map)
         if p is None:
@@ -54,6 +55,8 @@ class _SortChunks(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out, grad_probs, _grad_map):
         (row_map,) = ctx.saved_tensors
+        if grad_out is None:
+            return None, None, None, None
         lib = _lib.load()
         dev = grad_out.device
         g = grad_out.contiguous()
