@@ -28,6 +28,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}   # dense, published
 
+# HBM bytes per launch of the dominant kernel (forward grouped matmul, fc1/fc2 average) from rocprofv3
+# FETCH_SIZE + WRITE_SIZE, scaled by what the same counters read for the plain copy kernel of known size
+# (profiles/gmm_forward_mixtral_pmc.txt).  None where it has not been measured.
+TRAFFIC_BYTES_PER_LAUNCH = {"mixtral": None}
+
 WORKLOADS = {
     # name: (tokens, hidden, experts, topk, ffn, dtype, routing)
     "plumbing": dict(T=512, H=256, E=8, K=2, F=512, dtype="f32", routing="uniform",
@@ -118,6 +123,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="mixtral", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="after the steps, run the plain copy kernel over this many MiB three times "
+                         "(reference point for profiler byte counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one rank's expert path on ONE GPU (no collectives are part of this path); "
@@ -141,16 +149,23 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # timed region: exactly K steps, nothing else on the stream
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    tokens_per_s = cfg["T"] / (ms_per_step / 1e3)
+
+    # the same K steps again with every op bracketed by two events on its launch stream: per-kernel times
     with flop_counter.record(timing=True) as rec:
         t0 = time.perf_counter()
         for _ in range(args.steps):
             step()
         torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
-    tokens_per_s = cfg["T"] / (ms_per_step / 1e3)
+        ms_per_step_events = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # per-op breakdown from the events recorded on the launch stream inside the timed region
     kernels = {}
     for name, s in rec.summary().items():
         avg_ms = s["ms"] / s["calls"]
@@ -166,9 +181,12 @@ def main():
 
     peak = MFMA_PEAK_TFLOPS[cfg["dtype"]]
     dom = kernels["gmm_fwd"]          # the forward grouped matmul: fc1 and fc2 launches averaged
-    roofline = {"bound": "mfma", "kernel": "gmm16_kernel (NN, forward grouped matmul; fc1+fc2 averaged)"
-                if cfg["dtype"] == "bf16" else "gmm32_kernel", "achieved": dom["tflops"], "peak": peak,
-                "unit": "TFLOP/s", "frac": round(dom["tflops"] / peak, 4), "traffic": None}
+    roofline = {"bound": "mfma",
+                "kernel": "gmm16_fast_kernel<bf16, A reduction-contiguous, B column-contiguous> (forward grouped "
+                          "matmul; one launch each for fc1 and fc2, averaged)" if cfg["dtype"] == "bf16"
+                else "gmm32_kernel (forward grouped matmul, fp32)",
+                "achieved": dom["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": round(dom["tflops"] / peak, 4),
+                "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(args.workload)}
     for name in ("gmm_dx", "gmm_dw"):
         kernels[name]["frac_of_mfma_peak"] = round(kernels[name]["tflops"] / peak, 4)
     kernels["gmm_fwd"]["frac_of_mfma_peak"] = roofline["frac"]
@@ -184,6 +202,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step_with_event_timing": round(ms_per_step_events, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -195,6 +214,16 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    if args.copy_calibration:
+        from mindspeed_amd import _lib
+        lib = _lib.load()
+        n = args.copy_calibration << 20
+        src = torch.empty(n, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _lib.check(lib.ms_copy_bytes(_lib.stream_ptr(device), _lib.ptr(src), _lib.ptr(dst), n), "ms_copy_bytes")
+        torch.cuda.synchronize()
+        result["copy_calibration_bytes"] = n
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(result))
