@@ -25,11 +25,29 @@ namespace ms {
 namespace {
 
 // ---- schedule ------------------------------------------------------------------------
+// One entry per group.  With split_tails the last row tile of a group may be a smaller one (64 or 128
+// rows, the smallest that holds the remainder), so ragged groups do not pay for a whole extra tile; it
+// stays in the group's tile range, next to the full tiles of the same column panel, so the weight panel
+// it reads is being read by its neighbours at the same time.
+__device__ __forceinline__ int emit_rows(TileTable *table, int n, int &tiles, GroupEntry e, int tile_rows,
+                                         int num_col_tiles, int split_tails) {
+    const int rows = e.row_end - e.row_begin;
+    if (rows <= 0) return n;
+    e.tile_rows = tile_rows;
+    e.num_row_tiles = (rows + tile_rows - 1) / tile_rows;
+    const int rem = rows - (e.num_row_tiles - 1) * tile_rows;      // rows of the last tile, 1..tile_rows
+    e.tail_rows = !split_tails ? 0 : (rem <= 64 ? 64 : (rem <= 128 ? 128 : 0));
+    e.tile_begin = tiles;
+    tiles += e.num_row_tiles * num_col_tiles;
+    table->entries[n++] = e;
+    return n;
+}
+
 __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__restrict__ group_list,
                                                            int group_list_type, int group_type, int num_groups,
                                                            int m, int k, int tile_rows, int num_col_tiles,
-                                                           int64_t b_stride_group, int64_t c_stride_group,
-                                                           TileTable *table) {
+                                                           int split_tails, int64_t b_stride_group,
+                                                           int64_t c_stride_group, TileTable *table) {
     extern __shared__ int64_t gl[];
     for (int g = threadIdx.x; g < num_groups; g += blockDim.x) gl[g] = group_list[g];
     __syncthreads();
@@ -41,7 +59,7 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
         int64_t end = group_list_type == 0 ? gl[g] : prev + gl[g];
         end = end < prev ? prev : end;
         end = end > m ? m : end;
-        GroupEntry e;
+        GroupEntry e{};
         if (group_type == 0) {
             e.row_begin = static_cast<int>(prev);
             e.row_end = static_cast<int>(end);
@@ -57,30 +75,19 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
             e.b_off = 0;
             e.c_off = g * c_stride_group;
         }
-        e.num_row_tiles = (e.row_end - e.row_begin + tile_rows - 1) / tile_rows;
-        e.tile_begin = tiles;
-        tiles += e.num_row_tiles * num_col_tiles;
-        table->entries[n++] = e;
+        n = emit_rows(table, n, tiles, e, tile_rows, num_col_tiles, split_tails);
         prev = end;
     }
     if (group_type == 0 && prev < m) {  // rows past the last offset: zero-fill
-        GroupEntry e;
+        GroupEntry e{};
         e.row_begin = static_cast<int>(prev);
         e.row_end = m;
-        e.red_begin = 0;
-        e.red_end = 0;
-        e.b_off = 0;
-        e.c_off = 0;
-        e.num_row_tiles = (e.row_end - e.row_begin + tile_rows - 1) / tile_rows;
-        e.tile_begin = tiles;
-        tiles += e.num_row_tiles * num_col_tiles;
-        table->entries[n++] = e;
+        n = emit_rows(table, n, tiles, e, tile_rows, num_col_tiles, split_tails);
     }
     table->total_tiles = tiles;
     table->num_entries = n;
 }
 
-// ---- 16-bit MFMA kernel ------------------------------------------------------------------
 // 8 contiguous 16-bit elements starting at p; elements >= nvalid read as zero.
 __device__ __forceinline__ v16 load8(const uint16_t *p, int nvalid, bool vec_ok) {
     if (nvalid >= 8 && vec_ok && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) return *reinterpret_cast<const v16 *>(p);
@@ -169,7 +176,7 @@ __global__ __launch_bounds__(256) void gmm16_kernel(const GmmArgs p) {
     const int wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
 
-    const int row0 = tc.e.row_begin + tc.row_tile * BM;
+    const int row0 = tc.e.row_begin + tc.row_tile * tc.e.tile_rows;
     const int row_end = tc.e.row_end;
     const int col0 = tc.col_tile * BN;
     const int col_end = p.cols;
@@ -301,7 +308,7 @@ __global__ __launch_bounds__(256) void gmm32_kernel(const GmmArgs p) {
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int row0 = tc.e.row_begin + tc.row_tile * FM;
+    const int row0 = tc.e.row_begin + tc.row_tile * tc.e.tile_rows;
     const int row_end = tc.e.row_end;
     const int col0 = tc.col_tile * FN;
     const int col_end = p.cols;
@@ -376,7 +383,7 @@ __global__ __launch_bounds__(256) void gmm32_kernel(const GmmArgs p) {
 
 // ---- host -------------------------------------------------------------------------------
 size_t table_bytes(int64_t num_groups) {
-    return sizeof(TileTable) + static_cast<size_t>(num_groups + 1) * sizeof(GroupEntry);
+    return sizeof(TileTable) + static_cast<size_t>(num_groups + 2) * sizeof(GroupEntry);
 }
 
 template <int DT, int OUT>
@@ -455,18 +462,21 @@ extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int
     const int tile_rows = is32 ? FM : BM;
     const int tile_cols = is32 ? FN : BN;
     const int64_t num_col_tiles = ceil_div(n, tile_cols);
-    const int64_t row_tiles_bound = group_type == 0 ? ceil_div(m, tile_rows) + num_groups + 1
-                                                    : num_groups * ceil_div(k, tile_rows);
+    const int64_t row_tiles_bound = group_type == 0 ? ceil_div(m, tile_rows) + num_groups + 2
+                                                    : num_groups * (k / tile_rows + 1);
     const int64_t tiles_bound = row_tiles_bound * num_col_tiles;
     MS_REQUIRE(tiles_bound < (1ll << 30), MS_ERR_UNSUPPORTED, "ms_gmm: problem too large (%lld tiles)", (long long)tiles_bound);
 
     TileTable *table = static_cast<TileTable *>(workspace);
     const int64_t c_stride_group = k * y_stride_row;
-    hipLaunchKernelGGL(gmm_schedule_kernel, dim3(1), dim3(256), static_cast<size_t>(num_groups) * sizeof(int64_t), stream,
-                       group_list, group_list_type, group_type, static_cast<int>(num_groups), static_cast<int>(m),
-                       static_cast<int>(k), tile_rows, static_cast<int>(num_col_tiles), w_stride_group, c_stride_group,
-                       table);
-    MS_CHECK_LAUNCH("gmm_schedule_kernel");
+    auto schedule = [&](int split_tails) -> int {
+        hipLaunchKernelGGL(gmm_schedule_kernel, dim3(1), dim3(256), static_cast<size_t>(num_groups) * sizeof(int64_t),
+                           stream, group_list, group_list_type, group_type, static_cast<int>(num_groups),
+                           static_cast<int>(m), static_cast<int>(k), tile_rows, static_cast<int>(num_col_tiles),
+                           split_tails, w_stride_group, c_stride_group, table);
+        MS_CHECK_LAUNCH("gmm_schedule_kernel");
+        return MS_OK;
+    };
 
     GmmArgs args{};
     args.a = x;
@@ -483,6 +493,7 @@ extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int
     const unsigned grid = static_cast<unsigned>(ceil_div(tiles_bound, 8) * 8);
 
     if (is32) {
+        if (int rc = schedule(0)) return rc;
         if (accumulate)
             hipLaunchKernelGGL(gmm32_kernel<true>, dim3(grid), dim3(256), 0, stream, args);
         else
@@ -521,6 +532,7 @@ extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int
     const int64_t a_span = a_is_red ? 256 * a_stride_row : 64 * a_stride_red;
     const int64_t b_span = b_is_red ? 256 * b_stride_col : 64 * b_stride_red;
     fast = fast && a_span < (1ll << 30) && b_span < (1ll << 30);
+    if (int rc = schedule(fast ? 1 : 0)) return rc;
     if (fast) return launch_gmm16_fast(stream, args, dtype, out, a_is_red, b_is_red, grid);
     if (dtype == MS_BF16) {
         if (out == OUT_SAME) return launch16<MS_BF16, OUT_SAME>(stream, args, a_is_red, b_is_red, grid);

@@ -17,6 +17,8 @@ struct GroupEntry {
     int red_begin, red_end;  // reduction range of the group
     int tile_begin;          // first logical tile
     int num_row_tiles;
+    int tile_rows;           // rows per full tile
+    int tail_rows;           // rows of the group's last row tile if it is a smaller one (64 / 128), else 0
     int64_t b_off;           // element offset of the group's weight block
     int64_t c_off;           // element offset of the group's output block
 };
@@ -44,6 +46,7 @@ struct GmmArgs {
 struct TileCoord {
     GroupEntry e;
     int row_tile, col_tile;
+    int tile_rows;           // rows of this tile (the entry's tile_rows, or its tail_rows for the last row tile)
     bool valid;
 };
 
@@ -67,6 +70,7 @@ __device__ __forceinline__ TileCoord locate_tile(const TileTable *table) {
     const int r = logical - tc.e.tile_begin;
     tc.col_tile = r / tc.e.num_row_tiles;
     tc.row_tile = r - tc.col_tile * tc.e.num_row_tiles;
+    tc.tile_rows = (tc.e.tail_rows != 0 && tc.row_tile == tc.e.num_row_tiles - 1) ? tc.e.tail_rows : tc.e.tile_rows;
     tc.valid = true;
     return tc;
 }

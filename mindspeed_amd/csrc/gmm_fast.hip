@@ -2,7 +2,9 @@
 // 256-thread workgroup (2x2 wavefronts, 128x128 per wavefront = 4x4
 // v_mfma_f32_32x32x16), for problems whose pointers and strides allow 16-byte
 // vector access everywhere.  All edge handling is branch-free (clamped addresses,
-// zero masks on the reduction tail).
+// zero masks on the reduction tail).  The last row tile of a group may be a
+// 128x256 or 64x256 tile (1x4 wavefronts of 128x64 / 64x64) so that ragged
+// groups do not pay for a full 256-row tile; the tile table says which.
 //
 // LDS layout per operand tile
 //   * operand contiguous along the reduction dim in memory ("RED"): stored as
@@ -27,6 +29,7 @@
 // Every load therefore has a full K step (64 MFMAs per wavefront) to arrive, and the
 // vector memory path sees a steady request stream instead of one burst per step.
 #include <type_traits>
+#include <utility>
 
 #include "gmm_common.h"
 
@@ -41,12 +44,12 @@ __device__ __forceinline__ void sg() {
     if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, ID);
 }
 
-constexpr int kPitchT = 576;                      // row pitch of an outer-contiguous tile: 512 + 64 bytes
-constexpr int kRedTileBytes = 256 * 128;          // [256 outer][64 red] x 2 bytes
-constexpr int kOuterTileBytes = 64 * kPitchT;     // [64 red][256 outer] x 2 bytes, padded rows
-
-template <bool RED>
-constexpr int tile_bytes() { return RED ? kRedTileBytes : kOuterTileBytes; }
+// Bytes of one operand tile in LDS.  RED: [ROWS outer][64 reduction] x 2 bytes.  !RED: [64 reduction][ROWS outer]
+// x 2 bytes with 64 bytes of padding per row (pitch mod 256 == 64 keeps the transposing reads conflict-free).
+template <bool RED, int ROWS>
+constexpr int tile_bytes() { return RED ? ROWS * 128 : 64 * (ROWS * 2 + 64); }
+constexpr int kRedTileBytes = tile_bytes<true, 256>();
+constexpr int kOuterTileBytes = tile_bytes<false, 256>();
 
 constexpr int kStagePitch = 264;                          // epilogue staging: 128 x 2 bytes + 8 bytes pad
 constexpr int kStagePerWave = 128 * kStagePitch;          // one 128 x 128 16-bit block per wavefront
@@ -60,14 +63,19 @@ __device__ __forceinline__ uint2 lds_read_tr(const char *p) {
     return __builtin_bit_cast(uint2, v);
 }
 
-// One operand of the macro tile: global -> registers -> LDS, and LDS -> MFMA fragments.
-template <bool RED>
+// One operand of the macro tile (ROWS outer indices x 64 reduction indices):
+// global -> registers -> LDS, and LDS -> MFMA fragments.
+template <bool RED, int ROWS>
 struct Operand {
-    unsigned off[8];    // per-lane global byte offsets of the 8 loads, relative to the tile's base pointer
+    static constexpr int NL = ROWS / 32;          // 16-byte loads per lane per K step (8, 4 or 2)
+    static constexpr int PITCH = ROWS * 2 + 64;   // !RED: bytes per reduction row in LDS
+    static constexpr int CP = ROWS / 8;           // !RED: 16-byte chunks per reduction row
+    static constexpr int RP = 256 / CP;           // !RED: reduction rows covered by one load of the workgroup
+    unsigned off[NL];   // per-lane global byte offsets of the loads, relative to the tile's base pointer
     unsigned off0;      // !RED: offset of (reduction index 0, this lane's outer chunk), always valid
     unsigned st_off;    // byte offset of this lane's first LDS store inside the tile
     unsigned frag_off;  // byte offset of this lane's fragment reads inside the tile
-    v16 r[8];
+    v16 r[NL];
 
     // outer0: first outer index of the tile; outer_last: clamp bound (RED: last valid outer index,
     // !RED: last valid start of an 8-wide chunk); wave_outer: this wavefront's first outer index in the tile.
@@ -79,7 +87,7 @@ struct Operand {
             const int ck = tid & 7;
             const int row = tid >> 3;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
+            for (int i = 0; i < NL; ++i) {
                 int outer = outer0 + row + 32 * i;
                 outer = outer > outer_last ? outer_last : outer;
                 off[i] = static_cast<unsigned>((static_cast<int64_t>(outer - outer0) * stride_outer + ck * 8) * 2);
@@ -89,31 +97,31 @@ struct Operand {
             const int frow = lane & 31;
             frag_off = (wave_outer + frow) * 128 + (((lane >> 5) ^ swz(frow)) << 4);
         } else {
-            const int chunk = tid & 31;   // 16-byte chunk along the outer dim
-            const int rrow = tid >> 5;    // reduction row within a group of 8
+            const int chunk = tid % CP;   // 16-byte chunk along the outer dim
+            const int rrow = tid / CP;    // reduction row within one load of the workgroup
             int outer = outer0 + chunk * 8;
             outer = outer > outer_last ? outer_last : outer;
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                off[i] = static_cast<unsigned>((static_cast<int64_t>(i * 8 + rrow) * stride_red + (outer - outer0)) * 2);
+            for (int i = 0; i < NL; ++i)
+                off[i] = static_cast<unsigned>((static_cast<int64_t>(i * RP + rrow) * stride_red + (outer - outer0)) * 2);
             off0 = static_cast<unsigned>((outer - outer0) * 2);
-            st_off = rrow * kPitchT + chunk * 16;
+            st_off = rrow * PITCH + chunk * 16;
             // transposing read: in each group of 16 lanes, lane L supplies the 4-element segment at
             // (reduction L/4, outer 4*(L%4)) and receives reduction 0..3 of outer L.
             const int l16 = lane & 15;
             const int red = 8 * (lane >> 5) + (l16 >> 2);
             const int out = wave_outer + 16 * ((lane >> 4) & 1) + 4 * (l16 & 3);
-            frag_off = red * kPitchT + out * 2;
+            frag_off = red * PITCH + out * 2;
         }
     }
 
-    // base: pointer to element (outer0, red0) of the tile.  Loads i = 4h..4h+3 of this lane.
+    // base: pointer to element (outer0, red0) of the tile.  Loads i = h*NL/2 .. (h+1)*NL/2 - 1 of this lane.
     // TAIL: the tile may cross red_end, reduction indices >= nvalid (relative to red0) read as zero.
     template <bool TAIL>
     __device__ __forceinline__ void load_half(const char *base, int nvalid, int h) {
         const int tid = threadIdx.x;
 #pragma unroll
-        for (int i = 4 * h; i < 4 * h + 4; ++i) {
+        for (int i = h * (NL / 2); i < (h + 1) * (NL / 2); ++i) {
             if constexpr (!TAIL) {
                 r[i] = *reinterpret_cast<const v16 *>(base + off[i]);
             } else {
@@ -121,7 +129,7 @@ struct Operand {
                 // multiple of 8 on this path); !RED: one reduction index per load.  Masked-out lanes read a
                 // valid address (chunk 0 / reduction index 0) instead.
                 const int q = tid & 7;
-                const bool ok = RED ? (q * 8 < nvalid) : (i * 8 + (tid >> 5) < nvalid);
+                const bool ok = RED ? (q * 8 < nvalid) : (i * RP + tid / CP < nvalid);
                 const unsigned o = ok ? off[i] : (RED ? off[i] - q * 16 : off0);
                 const v16 v = *reinterpret_cast<const v16 *>(base + o);
                 const v16 z = {0u, 0u, 0u, 0u};
@@ -132,9 +140,9 @@ struct Operand {
 
     __device__ __forceinline__ void store_half(char *tile, int h) const {
 #pragma unroll
-        for (int i = 4 * h; i < 4 * h + 4; ++i) {
+        for (int i = h * (NL / 2); i < (h + 1) * (NL / 2); ++i) {
             if constexpr (RED) *reinterpret_cast<v16 *>(tile + st_off + i * 32 * 128) = r[i];
-            else *reinterpret_cast<v16 *>(tile + st_off + i * 8 * kPitchT) = r[i];
+            else *reinterpret_cast<v16 *>(tile + st_off + i * RP * PITCH) = r[i];
         }
     }
 
@@ -144,46 +152,60 @@ struct Operand {
         if constexpr (RED) {
             return *reinterpret_cast<const v16 *>(tile + (frag_off ^ ((kk * 2) << 4)) + t * 32 * 128);
         } else {
-            const char *p = tile + frag_off + kk * 16 * kPitchT + t * 64;
+            const char *p = tile + frag_off + kk * 16 * PITCH + t * 64;
             const uint2 lo = lds_read_tr(p);
-            const uint2 hi = lds_read_tr(p + 4 * kPitchT);
+            const uint2 hi = lds_read_tr(p + 4 * PITCH);
             return v16{lo.x, lo.y, hi.x, hi.y};
         }
     }
 };
 
-template <int DT, bool A_RED, bool B_RED, int OUT>
-__global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
-    extern __shared__ __attribute__((aligned(16))) char lds[];
-    constexpr int A_BYTES = tile_bytes<A_RED>();
-    constexpr int STAGE = A_BYTES + tile_bytes<B_RED>();
-    const TileCoord tc = locate_tile(p.table);
-    if (!tc.valid) return;
+// sched_group_barrier sequence for one phase: NM MFMAs with NRD LDS reads, NWR LDS writes and NLD global
+// loads spread evenly between them.
+constexpr int share(int total, int slots, int g) { return total * (g + 1) / slots - total * g / slots; }
+
+template <int NM, int NRD, int NWR, int NLD, int ID, int... G>
+__device__ __forceinline__ void interleave(std::integer_sequence<int, G...>) {
+    ((sg<SG_DS_RD, share(NRD, NM, G), ID>(), sg<SG_DS_WR, share(NWR, NM, G), ID>(),
+      sg<SG_VMEM_RD, share(NLD, NM, G), ID>(), sg<SG_MFMA, 1, ID>()),
+     ...);
+}
+
+// One macro tile of TBM x 256 outputs.  TBM = 256: 2x2 wavefronts of 128x128; TBM = 128 / 64: 1x4 wavefronts
+// of 128x64 / 64x64.
+template <int DT, bool A_RED, bool B_RED, int OUT, int TBM>
+__device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc, char *lds) {
+    constexpr int WAVES_M = TBM == 256 ? 2 : 1;
+    constexpr int WAVES_N = 4 / WAVES_M;
+    constexpr int TM = TBM / WAVES_M / 32;      // 32-row MFMA blocks per wavefront
+    constexpr int TN = BN / WAVES_N / 32;       // 32-column MFMA blocks per wavefront
+    constexpr int A_BYTES = tile_bytes<A_RED, TBM>();
+    constexpr int STAGE = A_BYTES + tile_bytes<B_RED, BN>();
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int hi = lane >> 5;
 
-    const int row0 = tc.e.row_begin + tc.row_tile * BM;
+    const int row0 = tc.e.row_begin + tc.row_tile * BM;   // all but the last row tile of a group are full
     const int row_end = tc.e.row_end;
     const int col0 = tc.col_tile * BN;
     const int col_end = p.cols;
     const int red_begin = tc.e.red_begin, red_end = tc.e.red_end;
 
-    f32x16 acc[4][4];
+    f32x16 acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    Operand<A_RED> la;
-    Operand<B_RED> lb;
-    la.init(p.a_stride_row, p.a_stride_red, row0, A_RED ? row_end - 1 : row_end - 8, wm * 128);
-    lb.init(p.b_stride_col, p.b_stride_red, col0, B_RED ? col_end - 1 : col_end - 8, wn * 128);
+    Operand<A_RED, TBM> la;
+    Operand<B_RED, BN> lb;
+    la.init(p.a_stride_row, p.a_stride_red, row0, A_RED ? row_end - 1 : row_end - 8, wm * TM * 32);
+    lb.init(p.b_stride_col, p.b_stride_red, col0, B_RED ? col_end - 1 : col_end - 8, wn * TN * 32);
     // uniform base pointers of element (outer0, red_begin); advanced by one K step per iteration
     const char *a_ptr = static_cast<const char *>(p.a) +
                         (static_cast<int64_t>(row0) * p.a_stride_row + static_cast<int64_t>(red_begin) * p.a_stride_red) * 2;
@@ -196,19 +218,18 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
     const int red_len = red_end - red_begin;
     const int nk = (red_len + BK - 1) / BK;
 
-    v16 af[2][4], bf[2][4];
+    v16 af[2][TM], bf[2][TN];
     auto read_frags = [&](const char *stage, int set, int kk) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            af[set][t] = la.frag(stage, kk, t);
-            bf[set][t] = lb.frag(stage + A_BYTES, kk, t);
-        }
+        for (int t = 0; t < TM; ++t) af[set][t] = la.frag(stage, kk, t);
+#pragma unroll
+        for (int t = 0; t < TN; ++t) bf[set][t] = lb.frag(stage + A_BYTES, kk, t);
     };
     auto mfmas = [&](int set, int i0, int i1) {
 #pragma unroll
         for (int i = i0; i < i1; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i][j] = mfma16<DT>(bf[set][j], af[set][i], acc[i][j]);
+            for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<DT>(bf[set][j], af[set][i], acc[i][j]);
     };
     // part p of a tile: p = 0,1 -> A halves, p = 2,3 -> B halves
     auto load_part = [&](auto tail_c, int part, int nvalid) {
@@ -243,8 +264,11 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
         read_frags(lds, 0, 0);
     }
 
-    // LDS fragment-read instructions per 16-MFMA phase (ds_read_b128 x4 or ds_read_b64_tr x8 per operand)
-    constexpr int NRD = (A_RED ? 4 : 8) + (B_RED ? 4 : 8);
+    // instruction counts of one phase (one 16-wide K slice)
+    constexpr int NM = TM * TN;                                        // MFMAs
+    constexpr int NRD = (A_RED ? TM : 2 * TM) + (B_RED ? TN : 2 * TN); // LDS fragment reads
+    constexpr int NLA = Operand<A_RED, TBM>::NL / 2;                   // loads / stores of an A part
+    constexpr int NLB = Operand<B_RED, BN>::NL / 2;                    // ... of a B part
 
     int kt = 0;
     // HAS1: tile kt+1 exists (it is in registers); HAS2: tile kt+2 exists; tail2_c: tile kt+2 is the last one.
@@ -261,47 +285,28 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
             const int set = kk & 1;
-#ifndef EXP_NOSTORE
             if constexpr (HAS1) store_part(nxt, kk);
-#endif
-#ifndef EXP_NOLOAD
             if constexpr (HAS2) load_part(tail2_c, kk, left2);
-#endif
-            if (kk < 3) {
+            if (kk < 2) {
                 read_frags(cur, set ^ 1, kk + 1);
-                mfmas(set, 0, 4);
-#pragma unroll
-                for (int g = 0; g < 8; ++g) {
-                    sg<SG_DS_RD, 1, 0>();
-                    sg<SG_MFMA, 1, 0>();
-                    if (g < 4) sg<SG_DS_WR, HAS1 ? 1 : 0, 0>(); else sg<SG_VMEM_RD, HAS2 ? 1 : 0, 0>();
-                    if (NRD == 16 || (NRD == 12 && (g & 1))) sg<SG_DS_RD, 1, 0>();
-                    sg<SG_MFMA, 1, 0>();
-                }
+                mfmas(set, 0, TM);
+                interleave<NM, NRD, HAS1 ? NLA : 0, HAS2 ? NLA : 0, 0>(std::make_integer_sequence<int, NM>{});
+                __builtin_amdgcn_sched_barrier(0);
+            } else if (kk == 2) {
+                read_frags(cur, set ^ 1, kk + 1);
+                mfmas(set, 0, TM);
+                interleave<NM, NRD, HAS1 ? NLB : 0, HAS2 ? NLB : 0, 0>(std::make_integer_sequence<int, NM>{});
                 __builtin_amdgcn_sched_barrier(0);
             } else {
-                mfmas(set, 0, 2);
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    sg<SG_DS_WR, HAS1 ? 1 : 0, 0>();
-                    sg<SG_MFMA, 1, 0>();
-                    sg<SG_VMEM_RD, HAS2 ? 1 : 0, 0>();
-                    sg<SG_MFMA, 1, 0>();
-                }
+                mfmas(set, 0, TM / 2);
+                interleave<NM / 2, 0, HAS1 ? NLB : 0, HAS2 ? NLB : 0, 0>(std::make_integer_sequence<int, NM / 2>{});
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr (HAS1) {
                     lds_barrier();
                     read_frags(nxt, 0, 0);
                 }
-                mfmas(set, 2, 4);
-                if constexpr (HAS1) {
-#pragma unroll
-                    for (int g = 0; g < 8; ++g) {
-                        sg<SG_DS_RD, NRD / 8, 1>();
-                        if (NRD == 12 && (g & 1)) sg<SG_DS_RD, 1, 1>();
-                        sg<SG_MFMA, 1, 1>();
-                    }
-                }
+                mfmas(set, TM / 2, TM);
+                if constexpr (HAS1) interleave<NM / 2, NRD, 0, 0, 1>(std::make_integer_sequence<int, NM / 2>{});
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -311,54 +316,59 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
     if (kt + 2 == nk) { k_step(std::true_type{}, std::false_type{}, std::false_type{}); ++kt; }
     if (kt + 1 == nk) { k_step(std::false_type{}, std::false_type{}, std::false_type{}); ++kt; }
 
-    // Epilogue.  acc[i][j][4*q+e] = C[row0 + wm*128 + i*32 + (lane&31)]
-    //                                [col0 + wn*128 + j*32 + 8*q + 4*(lane>>5) + e]
+    // Epilogue.  acc[i][j][4*q+e] = C[row0 + wm*TM*32 + i*32 + (lane&31)]
+    //                                [col0 + wn*TN*32 + j*32 + 8*q + 4*(lane>>5) + e]
     const int64_t ldc = p.c_stride_row;
+    constexpr int WR = TM * 32, WC = TN * 32;       // this wavefront's block of the tile
     if constexpr (OUT == OUT_SAME) {
-        // 16-bit output: each wavefront stages its 128x128 block in its own LDS region (row pitch 264
-        // bytes: conflict-free for the 8-byte column-slice writes and the row reads) and writes it out
-        // as 16 bytes per lane, 256 contiguous bytes per row.
+        // 16-bit output: each wavefront stages its block in its own LDS region (row pitch WC*2 + 8 bytes:
+        // conflict-free for the 8-byte column-slice writes and the row reads) and writes it out as 16 bytes
+        // per lane, WC*2 contiguous bytes per row.
+        constexpr int SP = WC * 2 + 8;
+        static_assert(WR * SP <= kStagePerWave, "staging region too small");
         __builtin_amdgcn_s_waitcnt(0xC07F);
         __builtin_amdgcn_s_barrier();          // every wavefront is done reading the operand stages
         char *stg = lds + wave * kStagePerWave;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     uint16_t h[4];
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         h[e] = DT == MS_BF16 ? BF16::from_float(acc[i][j][4 * q + e]) : FP16::from_float(acc[i][j][4 * q + e]);
-                    *reinterpret_cast<uint2 *>(stg + (i * 32 + (lane & 31)) * kStagePitch + (j * 32 + 8 * q + 4 * hi) * 2) =
+                    *reinterpret_cast<uint2 *>(stg + (i * 32 + (lane & 31)) * SP + (j * 32 + 8 * q + 4 * hi) * 2) =
                         *reinterpret_cast<uint2 *>(h);
                 }
         __builtin_amdgcn_s_waitcnt(0xC07F);    // own writes only: the region is private to this wavefront
-        const int chunk = lane & 15;           // 8 columns = 16 bytes
-        const int col = col0 + wn * 128 + chunk * 8;
+        constexpr int LPR = WC / 8;            // lanes per row (8 columns = 16 bytes each)
+        constexpr int RPP = 64 / LPR;          // rows per pass
+        const int chunk = lane % LPR;
+        const int col = col0 + wn * WC + chunk * 8;
         const bool col_ok = col < col_end;     // cols is a multiple of 8 on this path
         uint16_t *cbase = static_cast<uint16_t *>(p.c) + tc.e.c_off + col;
 #pragma unroll 4
-        for (int pass = 0; pass < 32; ++pass) {
-            const int r = pass * 4 + (lane >> 4);
-            const int row = row0 + wm * 128 + r;
-            const uint2 lo = *reinterpret_cast<const uint2 *>(stg + r * kStagePitch + chunk * 16);
-            const uint2 hi2 = *reinterpret_cast<const uint2 *>(stg + r * kStagePitch + chunk * 16 + 8);
+        for (int pass = 0; pass < WR / RPP; ++pass) {
+            const int r = pass * RPP + lane / LPR;
+            const int row = row0 + wm * WR + r;
+            const uint2 lo = *reinterpret_cast<const uint2 *>(stg + r * SP + chunk * 16);
+            const uint2 hi2 = *reinterpret_cast<const uint2 *>(stg + r * SP + chunk * 16 + 8);
             if (col_ok && row < row_end)
                 *reinterpret_cast<v16 *>(cbase + static_cast<int64_t>(row) * ldc) = v16{lo.x, lo.y, hi2.x, hi2.y};
         }
     } else {
         const bool full_cols = col0 + BN <= col_end;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int row = row0 + wm * 128 + i * 32 + (lane & 31);
+        for (int i = 0; i < TM; ++i) {
+            const int row = row0 + wm * WR + i * 32 + (lane & 31);
             if (row >= row_end) continue;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < TN; ++j) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const int col = col0 + wn * 128 + j * 32 + 8 * q + 4 * hi;
+                    const int col = col0 + wn * WC + j * 32 + 8 * q + 4 * hi;
                     if (!full_cols && col >= col_end) continue;   // cols is a multiple of 4 on this path
                     float *c = static_cast<float *>(p.c) + tc.e.c_off + static_cast<int64_t>(row) * ldc + col;
                     f32x4 o = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
@@ -368,6 +378,16 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
             }
         }
     }
+}
+
+template <int DT, bool A_RED, bool B_RED, int OUT>
+__global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const TileCoord tc = locate_tile(p.table);
+    if (!tc.valid) return;
+    if (tc.tile_rows == 256) gmm16_tile<DT, A_RED, B_RED, OUT, 256>(p, tc, lds);
+    else if (tc.tile_rows == 128) gmm16_tile<DT, A_RED, B_RED, OUT, 128>(p, tc, lds);
+    else gmm16_tile<DT, A_RED, B_RED, OUT, 64>(p, tc, lds);
 }
 
 template <int DT, int OUT>
