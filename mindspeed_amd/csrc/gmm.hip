@@ -37,8 +37,10 @@ __device__ __forceinline__ int emit_rows(TileTable *table, int n, int &tiles, Gr
     e.num_row_tiles = (rows + tile_rows - 1) / tile_rows;
     const int rem = rows - (e.num_row_tiles - 1) * tile_rows;      // rows of the last tile, 1..tile_rows
     e.tail_rows = !split_tails ? 0 : (rem <= 64 ? 64 : (rem <= 128 ? 128 : 0));
+    e.num_tiles = e.num_row_tiles * num_col_tiles;
+    e.share = (e.num_tiles + 7) >> 3;
     e.tile_begin = tiles;
-    tiles += e.num_row_tiles * num_col_tiles;
+    tiles += e.share;
     table->entries[n++] = e;
     return n;
 }
@@ -52,31 +54,41 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
     for (int g = threadIdx.x; g < num_groups; g += blockDim.x) gl[g] = group_list[g];
     __syncthreads();
     if (threadIdx.x != 0) return;
-    int64_t prev = 0;
     int tiles = 0;
     int n = 0;
-    for (int g = 0; g < num_groups; ++g) {
-        int64_t end = group_list_type == 0 ? gl[g] : prev + gl[g];
-        end = end < prev ? prev : end;
-        end = end > m ? m : end;
-        GroupEntry e{};
-        if (group_type == 0) {
-            e.row_begin = static_cast<int>(prev);
-            e.row_end = static_cast<int>(end);
-            e.red_begin = 0;
-            e.red_end = k;
-            e.b_off = g * b_stride_group;
-            e.c_off = 0;
-        } else {
-            e.row_begin = 0;
-            e.row_end = k;
-            e.red_begin = static_cast<int>(prev);
-            e.red_end = static_cast<int>(end);
-            e.b_off = 0;
-            e.c_off = g * c_stride_group;
+    int64_t prev = 0;
+    // Split on the reduction dim: a tile's cost is its group's reduction length, so groups with an
+    // above-average length are emitted first (they start early on every XCD), the short ones fill in after.
+    const int passes = group_type == 2 ? 2 : 1;
+    const int64_t mean_len = num_groups > 0 ? m / num_groups : 0;
+    for (int pass = 0; pass < passes; ++pass) {
+        prev = 0;
+        for (int g = 0; g < num_groups; ++g) {
+            int64_t end = group_list_type == 0 ? gl[g] : prev + gl[g];
+            end = end < prev ? prev : end;
+            end = end > m ? m : end;
+            const bool is_long = end - prev >= mean_len;
+            if (passes == 1 || is_long == (pass == 0)) {
+                GroupEntry e{};
+                if (group_type == 0) {
+                    e.row_begin = static_cast<int>(prev);
+                    e.row_end = static_cast<int>(end);
+                    e.red_begin = 0;
+                    e.red_end = k;
+                    e.b_off = g * b_stride_group;
+                    e.c_off = 0;
+                } else {
+                    e.row_begin = 0;
+                    e.row_end = k;
+                    e.red_begin = static_cast<int>(prev);
+                    e.red_end = static_cast<int>(end);
+                    e.b_off = 0;
+                    e.c_off = g * c_stride_group;
+                }
+                n = emit_rows(table, n, tiles, e, tile_rows, num_col_tiles, split_tails);
+            }
+            prev = end;
         }
-        n = emit_rows(table, n, tiles, e, tile_rows, num_col_tiles, split_tails);
-        prev = end;
     }
     if (group_type == 0 && prev < m) {  // rows past the last offset: zero-fill
         GroupEntry e{};
@@ -84,7 +96,7 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
         e.row_end = m;
         n = emit_rows(table, n, tiles, e, tile_rows, num_col_tiles, split_tails);
     }
-    table->total_tiles = tiles;
+    table->slots_per_xcd = tiles;
     table->num_entries = n;
 }
 
@@ -490,7 +502,7 @@ extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int
     args.c_stride_row = y_stride_row;
     args.cols = static_cast<int>(n);
     args.num_col_tiles = static_cast<int>(num_col_tiles);
-    const unsigned grid = static_cast<unsigned>(ceil_div(tiles_bound, 8) * 8);
+    const unsigned grid = static_cast<unsigned>((ceil_div(tiles_bound, 8) + num_groups + 2) * 8);
 
     if (is32) {
         if (int rc = schedule(0)) return rc;

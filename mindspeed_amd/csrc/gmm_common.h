@@ -15,16 +15,18 @@ constexpr int kMaxGroups = 4096;
 struct GroupEntry {
     int row_begin, row_end;  // output rows of the group
     int red_begin, red_end;  // reduction range of the group
-    int tile_begin;          // first logical tile
+    int tile_begin;          // first slot of this group in every XCD's slot sequence
     int num_row_tiles;
     int tile_rows;           // rows per full tile
     int tail_rows;           // rows of the group's last row tile if it is a smaller one (64 / 128), else 0
+    int num_tiles;           // num_row_tiles * column tiles
+    int share;               // ceil(num_tiles / 8): tiles of this group handled by each XCD
     int64_t b_off;           // element offset of the group's weight block
     int64_t c_off;           // element offset of the group's output block
 };
 
 struct TileTable {
-    int total_tiles;
+    int slots_per_xcd;       // sum of the entries' shares
     int num_entries;
     int pad[6];
     GroupEntry entries[1];
@@ -50,24 +52,25 @@ struct TileCoord {
     bool valid;
 };
 
-// Map this workgroup to its logical tile (XCD-aware, see file header).
+// Map this workgroup to its tile.  Workgroup b runs on XCD b % 8 (round-robin dispatch) and takes slot
+// b / 8 of that XCD's slot sequence.  Every XCD walks the groups in the same order and owns one contiguous
+// eighth of each group's tiles (row-tile-fastest inside a column panel), so concurrently running
+// workgroups of an XCD share operand panels in that XCD's L2, and every XCD gets an equal part of every
+// group however unequal the groups are.
 __device__ __forceinline__ TileCoord locate_tile(const TileTable *table) {
     TileCoord tc;
     tc.valid = false;
-    const int total = table->total_tiles;
-    const int per_xcd = (total + 7) >> 3;
     const int xcd = blockIdx.x & 7;
     const int slot = blockIdx.x >> 3;
-    if (slot >= per_xcd) return tc;
-    const int logical = xcd * per_xcd + slot;
-    if (logical >= total) return tc;
-    int lo = 0, hi = table->num_entries;  // last entry with tile_begin <= logical
+    if (slot >= table->slots_per_xcd) return tc;
+    int lo = 0, hi = table->num_entries;  // last entry with tile_begin <= slot
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
-        if (table->entries[mid].tile_begin <= logical) lo = mid; else hi = mid;
+        if (table->entries[mid].tile_begin <= slot) lo = mid; else hi = mid;
     }
     tc.e = table->entries[lo];
-    const int r = logical - tc.e.tile_begin;
+    const int r = xcd * tc.e.share + (slot - tc.e.tile_begin);
+    if (r >= tc.e.num_tiles) return tc;
     tc.col_tile = r / tc.e.num_row_tiles;
     tc.row_tile = r - tc.col_tile * tc.e.num_row_tiles;
     tc.tile_rows = (tc.e.tail_rows != 0 && tc.row_tile == tc.e.num_row_tiles - 1) ? tc.e.tail_rows : tc.e.tile_rows;
