@@ -29,6 +29,7 @@ struct TileTable {
     int slots_per_xcd;       // sum of the entries' shares
     int num_entries;
     int pad[6];
+    int zeros[8];            // always zero: source of out-of-range operand chunks (holds an aligned 16-byte block)
     GroupEntry entries[1];
 };
 

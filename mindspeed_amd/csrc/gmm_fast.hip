@@ -171,6 +171,224 @@ __device__ __forceinline__ void interleave(std::integer_sequence<int, G...>) {
      ...);
 }
 
+// ---- ring-buffered variant of the 256-row tile: global -> LDS transfers without a register stage ----------
+//
+// global_load_lds_dwordx4 moves 16 bytes per lane from per-lane global addresses straight into LDS, where one
+// wavefront's 64 lanes fill 1 KB of consecutive bytes.  The LDS position of a lane is therefore fixed and the
+// bank-conflict-avoiding swizzle is applied on the global side: the lane that owns LDS chunk c of a row
+// fetches the memory chunk that the swizzle maps to c.  With no staging registers and no LDS store
+// instructions the K loop can keep several tiles in flight: a ring of kRing stages of 32 reduction indices
+// (16 KB per operand), tile kt+4 being requested while tile kt is multiplied, so every transfer has more than
+// three K steps to arrive.
+//   RED operand:  [256 outer][32 reduction], 64-byte rows, chunk c of row r holds memory chunk c ^ ((r >> 2) & 3)
+//   !RED operand: [32 reduction][256 outer], 512-byte rows, chunk c of row r holds memory chunk c ^ ((r & 3) << 2)
+// (the first keeps 16 consecutive rows of one chunk column on 16 different bank groups for ds_read_b128, the
+// second keeps the four rows of one ds_read_b64_tr_b16 group on four different 64-byte bank groups).
+constexpr int KS = 32;                        // reduction indices per ring stage
+constexpr int kRing = 5;
+constexpr int kRingTile = 256 * KS * 2;       // bytes of one operand in one stage
+constexpr int kRingStage = 2 * kRingTile;
+constexpr int kRingBytes = kRing * kRingStage;
+constexpr int kXfers = kRingTile / 4 / 1024;  // 1 KB transfers per wavefront, operand and stage (4)
+
+constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | (lgkm << 8); }
+
+using global_cptr = const char __attribute__((address_space(1))) *;
+using lds_ptr = char __attribute__((address_space(3))) *;
+
+template <bool RED>
+struct RingOperand {
+    unsigned off[kXfers];   // per-lane global byte offsets of this wavefront's transfers, relative to the tile base
+    int key[kXfers];        // reduction index (relative to the tile) whose validity decides transfer i of this lane
+    unsigned frag_off;      // byte offset of this lane's fragment reads inside the operand tile
+    unsigned tsel[4];       // !RED: swizzled 64-byte column-group offset of fragment t
+
+    __device__ __forceinline__ void init(int64_t stride_outer, int64_t stride_red, int outer0, int outer_last,
+                                         int wave_outer, int wave) {
+        const int lane = threadIdx.x & 63;
+        if constexpr (RED) {
+            const int cg = (lane & 3) ^ ((lane >> 4) & 3);   // memory chunk of this lane: c ^ ((row >> 2) & 3)
+#pragma unroll
+            for (int i = 0; i < kXfers; ++i) {
+                const int row = (wave * kXfers + i) * 16 + (lane >> 2);
+                int outer = outer0 + row;
+                outer = outer > outer_last ? outer_last : outer;
+                off[i] = static_cast<unsigned>((static_cast<int64_t>(outer - outer0) * stride_outer + cg * 8) * 2);
+                key[i] = cg * 8;
+            }
+            const int frow = lane & 31;
+            frag_off = (wave_outer + frow) * 64 + (((lane >> 5) ^ ((frow >> 2) & 3)) << 4);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) tsel[t] = 0;
+        } else {
+#pragma unroll
+            for (int i = 0; i < kXfers; ++i) {
+                const int rr = (wave * kXfers + i) * 2 + (lane >> 5);
+                const int cg = (lane & 31) ^ ((rr & 3) << 2);
+                int outer = outer0 + cg * 8;
+                outer = outer > outer_last ? outer_last : outer;
+                off[i] = static_cast<unsigned>((static_cast<int64_t>(rr) * stride_red + (outer - outer0)) * 2);
+                key[i] = rr;
+            }
+            // transposing read: in each group of 16 lanes, lane L supplies the 4-element segment at
+            // (reduction L/4, outer 4*(L%4)) and receives reduction 0..3 of outer L.
+            const int l16 = lane & 15;
+            const int sw = l16 >> 2;
+            const int red = 8 * (lane >> 5) + sw;
+            frag_off = red * 512 + wave_outer * 2 + 32 * ((lane >> 4) & 1) + 8 * (l16 & 3);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) tsel[t] = (t ^ sw) << 6;
+        }
+    }
+
+    // Request transfer i of this wavefront's part of one tile.  base: pointer to element (outer0, first
+    // reduction index of the tile), uniform; dst: LDS byte address of this wavefront's part of the operand's
+    // stage; nvalid: reduction indices of the tile that lie inside the group (<= 0 for a tile past the end,
+    // >= KS for a whole one).  Lanes whose data lies outside fetch from a block of zeros instead, so every
+    // tile costs the same number of transfers whatever it holds: the wait counters of the K loop rely on that.
+    // Written as inline assembly on purpose: the compiler then does not know that LDS is being written
+    // behind its back and leaves all waiting on these transfers to the explicit s_waitcnt of the K loop
+    // (it would otherwise drain them before every transposing LDS read).  M0 carries the LDS address; no
+    // other code in these kernels uses M0.
+    __device__ __forceinline__ void request(int i, const char *base, unsigned dst, int nvalid, const char *zeros) const {
+        const char *src = key[i] < nvalid ? base + off[i] : zeros;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                     :: "s"(dst + i * 1024), "v"(src) : "memory");
+    }
+
+    // Fragment t of 16-wide slice kk of the tile at `tile`.
+    __device__ __forceinline__ v16 frag(const char *tile, int kk, int t) const {
+        if constexpr (RED) {
+            return *reinterpret_cast<const v16 *>(tile + (frag_off ^ (kk << 5)) + t * 32 * 64);
+        } else {
+            const char *p = tile + frag_off + tsel[t] + kk * 16 * 512;
+            const uint2 lo = lds_read_tr(p);
+            const uint2 hi = lds_read_tr(p + 4 * 512);
+            return v16{lo.x, lo.y, hi.x, hi.y};
+        }
+    }
+};
+
+// Which operand layouts take the ring: both operands contiguous along their outer dim (the weight-gradient
+// product x^T dy).  There every transfer covers whole 512-byte memory rows, and the register-staged loop is
+// at its slowest because both operands go through the slower transposing reads on top of the LDS stores.
+// An operand contiguous along the reduction dim would be fetched as 64-byte half lines (32 reduction
+// indices per stage), which doubles its request count at L2; measured, those products run a few percent
+// slower on the ring than on the register-staged loop, so they stay there.
+template <bool A_RED, bool B_RED>
+constexpr bool use_ring() { return !A_RED && !B_RED; }
+
+template <int DT, bool A_RED, bool B_RED>
+__device__ __forceinline__ void ring_k_loop(const GmmArgs &p, const TileCoord &tc, char *lds, int row0, int col0,
+                                            f32x16 (&acc)[4][4]) {
+    constexpr int TM = 4, TN = 4;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int red_begin = tc.e.red_begin;
+    const int red_len = tc.e.red_end - red_begin;
+    const int nk = (red_len + KS - 1) / KS;
+    if (nk <= 0) return;
+
+    RingOperand<A_RED> la;
+    RingOperand<B_RED> lb;
+    la.init(p.a_stride_row, p.a_stride_red, row0, A_RED ? tc.e.row_end - 1 : tc.e.row_end - 8, wm * 128, wave);
+    lb.init(p.b_stride_col, p.b_stride_red, col0, B_RED ? p.cols - 1 : p.cols - 8, wn * 128, wave);
+    const char *a_ptr = static_cast<const char *>(p.a) +
+                        (static_cast<int64_t>(row0) * p.a_stride_row + static_cast<int64_t>(red_begin) * p.a_stride_red) * 2;
+    const char *b_ptr = static_cast<const char *>(p.b) +
+                        (tc.e.b_off + static_cast<int64_t>(col0) * p.b_stride_col +
+                         static_cast<int64_t>(red_begin) * p.b_stride_red) * 2;
+    const int64_t a_step = p.a_stride_red * KS * 2;
+    const int64_t b_step = p.b_stride_red * KS * 2;
+    const char *zeros = reinterpret_cast<const char *>((reinterpret_cast<uintptr_t>(p.table->zeros) + 15) & ~uintptr_t(15));
+
+    const unsigned lds0 = static_cast<unsigned>(reinterpret_cast<uintptr_t>((lds_ptr)lds));
+    // Tiles are requested in order, one per K step plus kRing - 1 up front, and the sequence simply runs on
+    // past the last tile (all-zero tiles that nobody multiplies): the number of transfers in flight is then the
+    // same at every step and one wait count serves the whole loop.
+    int left = red_len;        // reduction indices from the next requested tile's start to the group's end
+    int issue_stage = 0;       // ring stage of the next request
+    // transfer g = 0..7 of the next tile: 0-3 operand A, 4-7 operand B
+    auto request_part = [&](int g) {
+        const unsigned dst = lds0 + issue_stage * kRingStage + wave * (kXfers * 1024);
+        if (g < kXfers) la.request(g, a_ptr, dst, left, zeros);
+        else lb.request(g - kXfers, b_ptr, dst + kRingTile, left, zeros);
+    };
+    auto request_done = [&]() {
+        a_ptr += a_step;
+        b_ptr += b_step;
+        left -= KS;
+        issue_stage = issue_stage + 1 == kRing ? 0 : issue_stage + 1;
+    };
+
+    v16 af[2][TM], bf[2][TN];
+    auto read_frags = [&](const char *stage, int set, int kk) {
+#pragma unroll
+        for (int t = 0; t < TM; ++t) af[set][t] = la.frag(stage, kk, t);
+#pragma unroll
+        for (int t = 0; t < TN; ++t) bf[set][t] = lb.frag(stage + kRingTile, kk, t);
+    };
+    auto mfmas = [&](int set, int i0, int i1) {
+#pragma unroll
+        for (int i = i0; i < i1; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<DT>(bf[set][j], af[set][i], acc[i][j]);
+    };
+    // Wait until only the kRing - 2 most recently requested tiles (2 * kXfers transfers each) are still in
+    // flight, and for this wavefront's LDS reads; then meet the other wavefronts.
+    auto arrive = [&]() {
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm((kRing - 2) * 2 * kXfers, 0));
+        __builtin_amdgcn_s_barrier();
+    };
+
+    for (int t = 0; t < kRing - 1; ++t) {
+#pragma unroll
+        for (int g = 0; g < 2 * kXfers; ++g) request_part(g);
+        request_done();
+    }
+    arrive();
+    read_frags(lds, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+
+    constexpr int NM = TM * TN;
+    constexpr int NRD = (A_RED ? TM : 2 * TM) + (B_RED ? TN : 2 * TN);
+    int cur_stage = 0;
+    // One K step of 32 reduction indices = two 16-wide slices.
+    for (int kt = 0; kt < nk; ++kt) {
+        const char *cur = lds + cur_stage * kRingStage;
+        cur_stage = cur_stage + 1 == kRing ? 0 : cur_stage + 1;
+        const char *nxt = lds + cur_stage * kRingStage;
+        // slice 0: eight groups of { one transfer request for tile kt + kRing - 1 (into the stage that tile
+        // kt - 1 occupied: free, every wavefront finished reading it before the barrier of the previous
+        // step), the slice-1 fragments of one 32-row block of each operand (first four groups), two MFMAs }
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            request_part(g);
+            if (g < 4) {
+                af[1][g] = la.frag(cur, 1, g);
+                bf[1][g] = lb.frag(cur + kRingTile, 1, g);
+            }
+#pragma unroll
+            for (int u = 2 * g; u < 2 * g + 2; ++u)
+                acc[u / TN][u % TN] = mfma16<DT>(bf[0][u % TN], af[0][u / TN], acc[u / TN][u % TN]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        request_done();
+        // slice 1: the barrier sits between the two halves of its MFMAs; after it tile kt + 1 is complete
+        // in LDS (after the last step that is an all-zero tile, read and never used)
+        mfmas(1, 0, TM / 2);
+        __builtin_amdgcn_sched_barrier(0);
+        arrive();
+        read_frags(nxt, 0, 0);
+        mfmas(1, TM / 2, TM);
+        interleave<NM / 2, NRD, 0, 0, 1>(std::make_integer_sequence<int, NM / 2>{});
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // the transfers of the trailing all-zero tiles must have landed before the stages are reused
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+}
+
 // One macro tile of TBM x 256 outputs.  TBM = 256: 2x2 wavefronts of 128x128; TBM = 128 / 64: 1x4 wavefronts
 // of 128x64 / 64x64.
 template <int DT, bool A_RED, bool B_RED, int OUT, int TBM>
@@ -202,119 +420,123 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    Operand<A_RED, TBM> la;
-    Operand<B_RED, BN> lb;
-    la.init(p.a_stride_row, p.a_stride_red, row0, A_RED ? row_end - 1 : row_end - 8, wm * TM * 32);
-    lb.init(p.b_stride_col, p.b_stride_red, col0, B_RED ? col_end - 1 : col_end - 8, wn * TN * 32);
-    // uniform base pointers of element (outer0, red_begin); advanced by one K step per iteration
-    const char *a_ptr = static_cast<const char *>(p.a) +
-                        (static_cast<int64_t>(row0) * p.a_stride_row + static_cast<int64_t>(red_begin) * p.a_stride_red) * 2;
-    const char *b_ptr = static_cast<const char *>(p.b) +
-                        (tc.e.b_off + static_cast<int64_t>(col0) * p.b_stride_col +
-                         static_cast<int64_t>(red_begin) * p.b_stride_red) * 2;
-    const int64_t a_step = p.a_stride_red * BK * 2;
-    const int64_t b_step = p.b_stride_red * BK * 2;
+    if constexpr (TBM == 256 && use_ring<A_RED, B_RED>()) {
+        ring_k_loop<DT, A_RED, B_RED>(p, tc, lds, row0, col0, acc);
+    } else {
+        Operand<A_RED, TBM> la;
+        Operand<B_RED, BN> lb;
+        la.init(p.a_stride_row, p.a_stride_red, row0, A_RED ? row_end - 1 : row_end - 8, wm * TM * 32);
+        lb.init(p.b_stride_col, p.b_stride_red, col0, B_RED ? col_end - 1 : col_end - 8, wn * TN * 32);
+        // uniform base pointers of element (outer0, red_begin); advanced by one K step per iteration
+        const char *a_ptr = static_cast<const char *>(p.a) +
+                            (static_cast<int64_t>(row0) * p.a_stride_row + static_cast<int64_t>(red_begin) * p.a_stride_red) * 2;
+        const char *b_ptr = static_cast<const char *>(p.b) +
+                            (tc.e.b_off + static_cast<int64_t>(col0) * p.b_stride_col +
+                             static_cast<int64_t>(red_begin) * p.b_stride_red) * 2;
+        const int64_t a_step = p.a_stride_red * BK * 2;
+        const int64_t b_step = p.b_stride_red * BK * 2;
 
-    const int red_len = red_end - red_begin;
-    const int nk = (red_len + BK - 1) / BK;
+        const int red_len = red_end - red_begin;
+        const int nk = (red_len + BK - 1) / BK;
 
-    v16 af[2][TM], bf[2][TN];
-    auto read_frags = [&](const char *stage, int set, int kk) {
-#pragma unroll
-        for (int t = 0; t < TM; ++t) af[set][t] = la.frag(stage, kk, t);
-#pragma unroll
-        for (int t = 0; t < TN; ++t) bf[set][t] = lb.frag(stage + A_BYTES, kk, t);
-    };
-    auto mfmas = [&](int set, int i0, int i1) {
-#pragma unroll
-        for (int i = i0; i < i1; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<DT>(bf[set][j], af[set][i], acc[i][j]);
-    };
-    // part p of a tile: p = 0,1 -> A halves, p = 2,3 -> B halves
-    auto load_part = [&](auto tail_c, int part, int nvalid) {
-        constexpr bool TAIL = decltype(tail_c)::value;
-        if (part < 2) la.template load_half<TAIL>(a_ptr, nvalid, part);
-        else lb.template load_half<TAIL>(b_ptr, nvalid, part - 2);
-    };
-    auto store_part = [&](char *stage, int part) {
-        if (part < 2) la.store_half(stage, part);
-        else lb.store_half(stage + A_BYTES, part - 2);
-    };
-    auto lds_barrier = [&]() {
-        __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0) only: global loads stay in flight
-        __builtin_amdgcn_s_barrier();
-    };
+        v16 af[2][TM], bf[2][TN];
+        auto read_frags = [&](const char *stage, int set, int kk) {
+    #pragma unroll
+            for (int t = 0; t < TM; ++t) af[set][t] = la.frag(stage, kk, t);
+    #pragma unroll
+            for (int t = 0; t < TN; ++t) bf[set][t] = lb.frag(stage + A_BYTES, kk, t);
+        };
+        auto mfmas = [&](int set, int i0, int i1) {
+    #pragma unroll
+            for (int i = i0; i < i1; ++i)
+    #pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<DT>(bf[set][j], af[set][i], acc[i][j]);
+        };
+        // part p of a tile: p = 0,1 -> A halves, p = 2,3 -> B halves
+        auto load_part = [&](auto tail_c, int part, int nvalid) {
+            constexpr bool TAIL = decltype(tail_c)::value;
+            if (part < 2) la.template load_half<TAIL>(a_ptr, nvalid, part);
+            else lb.template load_half<TAIL>(b_ptr, nvalid, part - 2);
+        };
+        auto store_part = [&](char *stage, int part) {
+            if (part < 2) la.store_half(stage, part);
+            else lb.store_half(stage + A_BYTES, part - 2);
+        };
+        auto lds_barrier = [&]() {
+            __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0) only: global loads stay in flight
+            __builtin_amdgcn_s_barrier();
+        };
 
-    if (nk > 0) {
-        // tile 0 -> LDS stage 0; tile 1 -> registers.  Both use the masked loads (whose results are
-        // consumed at once), so no load is outstanding when the steady-state loop is entered and the
-        // loop's own issue order alone decides how long each of its waits has to be.
-#pragma unroll
-        for (int part = 0; part < 4; ++part) load_part(std::true_type{}, part, red_len);
-#pragma unroll
-        for (int part = 0; part < 4; ++part) store_part(lds, part);
-        if (nk > 1) {
-            a_ptr += a_step;
-            b_ptr += b_step;
-#pragma unroll
-            for (int part = 0; part < 4; ++part) load_part(std::true_type{}, part, red_len - BK);
-        }
-        lds_barrier();
-        read_frags(lds, 0, 0);
-    }
-
-    // instruction counts of one phase (one 16-wide K slice)
-    constexpr int NM = TM * TN;                                        // MFMAs
-    constexpr int NRD = (A_RED ? TM : 2 * TM) + (B_RED ? TN : 2 * TN); // LDS fragment reads
-    constexpr int NLA = Operand<A_RED, TBM>::NL / 2;                   // loads / stores of an A part
-    constexpr int NLB = Operand<B_RED, BN>::NL / 2;                    // ... of a B part
-
-    int kt = 0;
-    // HAS1: tile kt+1 exists (it is in registers); HAS2: tile kt+2 exists; tail2_c: tile kt+2 is the last one.
-    auto k_step = [&](auto has1_c, auto has2_c, auto tail2_c) {
-        constexpr bool HAS1 = decltype(has1_c)::value;
-        constexpr bool HAS2 = decltype(has2_c)::value;
-        const char *cur = lds + (kt & 1) * STAGE;
-        char *nxt = lds + ((kt + 1) & 1) * STAGE;
-        if constexpr (HAS2) {
-            a_ptr += a_step;
-            b_ptr += b_step;
-        }
-        const int left2 = red_len - (kt + 2) * BK;
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            const int set = kk & 1;
-            if constexpr (HAS1) store_part(nxt, kk);
-            if constexpr (HAS2) load_part(tail2_c, kk, left2);
-            if (kk < 2) {
-                read_frags(cur, set ^ 1, kk + 1);
-                mfmas(set, 0, TM);
-                interleave<NM, NRD, HAS1 ? NLA : 0, HAS2 ? NLA : 0, 0>(std::make_integer_sequence<int, NM>{});
-                __builtin_amdgcn_sched_barrier(0);
-            } else if (kk == 2) {
-                read_frags(cur, set ^ 1, kk + 1);
-                mfmas(set, 0, TM);
-                interleave<NM, NRD, HAS1 ? NLB : 0, HAS2 ? NLB : 0, 0>(std::make_integer_sequence<int, NM>{});
-                __builtin_amdgcn_sched_barrier(0);
-            } else {
-                mfmas(set, 0, TM / 2);
-                interleave<NM / 2, 0, HAS1 ? NLB : 0, HAS2 ? NLB : 0, 0>(std::make_integer_sequence<int, NM / 2>{});
-                __builtin_amdgcn_sched_barrier(0);
-                if constexpr (HAS1) {
-                    lds_barrier();
-                    read_frags(nxt, 0, 0);
-                }
-                mfmas(set, TM / 2, TM);
-                if constexpr (HAS1) interleave<NM / 2, NRD, 0, 0, 1>(std::make_integer_sequence<int, NM / 2>{});
-                __builtin_amdgcn_sched_barrier(0);
+        if (nk > 0) {
+            // tile 0 -> LDS stage 0; tile 1 -> registers.  Both use the masked loads (whose results are
+            // consumed at once), so no load is outstanding when the steady-state loop is entered and the
+            // loop's own issue order alone decides how long each of its waits has to be.
+    #pragma unroll
+            for (int part = 0; part < 4; ++part) load_part(std::true_type{}, part, red_len);
+    #pragma unroll
+            for (int part = 0; part < 4; ++part) store_part(lds, part);
+            if (nk > 1) {
+                a_ptr += a_step;
+                b_ptr += b_step;
+    #pragma unroll
+                for (int part = 0; part < 4; ++part) load_part(std::true_type{}, part, red_len - BK);
             }
+            lds_barrier();
+            read_frags(lds, 0, 0);
         }
-    };
-    for (; kt + 3 < nk; ++kt) k_step(std::true_type{}, std::true_type{}, std::false_type{});
-    if (kt + 3 == nk) { k_step(std::true_type{}, std::true_type{}, std::true_type{}); ++kt; }
-    if (kt + 2 == nk) { k_step(std::true_type{}, std::false_type{}, std::false_type{}); ++kt; }
-    if (kt + 1 == nk) { k_step(std::false_type{}, std::false_type{}, std::false_type{}); ++kt; }
+
+        // instruction counts of one phase (one 16-wide K slice)
+        constexpr int NM = TM * TN;                                        // MFMAs
+        constexpr int NRD = (A_RED ? TM : 2 * TM) + (B_RED ? TN : 2 * TN); // LDS fragment reads
+        constexpr int NLA = Operand<A_RED, TBM>::NL / 2;                   // loads / stores of an A part
+        constexpr int NLB = Operand<B_RED, BN>::NL / 2;                    // ... of a B part
+
+        int kt = 0;
+        // HAS1: tile kt+1 exists (it is in registers); HAS2: tile kt+2 exists; tail2_c: tile kt+2 is the last one.
+        auto k_step = [&](auto has1_c, auto has2_c, auto tail2_c) {
+            constexpr bool HAS1 = decltype(has1_c)::value;
+            constexpr bool HAS2 = decltype(has2_c)::value;
+            const char *cur = lds + (kt & 1) * STAGE;
+            char *nxt = lds + ((kt + 1) & 1) * STAGE;
+            if constexpr (HAS2) {
+                a_ptr += a_step;
+                b_ptr += b_step;
+            }
+            const int left2 = red_len - (kt + 2) * BK;
+    #pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const int set = kk & 1;
+                if constexpr (HAS1) store_part(nxt, kk);
+                if constexpr (HAS2) load_part(tail2_c, kk, left2);
+                if (kk < 2) {
+                    read_frags(cur, set ^ 1, kk + 1);
+                    mfmas(set, 0, TM);
+                    interleave<NM, NRD, HAS1 ? NLA : 0, HAS2 ? NLA : 0, 0>(std::make_integer_sequence<int, NM>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                } else if (kk == 2) {
+                    read_frags(cur, set ^ 1, kk + 1);
+                    mfmas(set, 0, TM);
+                    interleave<NM, NRD, HAS1 ? NLB : 0, HAS2 ? NLB : 0, 0>(std::make_integer_sequence<int, NM>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                } else {
+                    mfmas(set, 0, TM / 2);
+                    interleave<NM / 2, 0, HAS1 ? NLB : 0, HAS2 ? NLB : 0, 0>(std::make_integer_sequence<int, NM / 2>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (HAS1) {
+                        lds_barrier();
+                        read_frags(nxt, 0, 0);
+                    }
+                    mfmas(set, TM / 2, TM);
+                    if constexpr (HAS1) interleave<NM / 2, NRD, 0, 0, 1>(std::make_integer_sequence<int, NM / 2>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        for (; kt + 3 < nk; ++kt) k_step(std::true_type{}, std::true_type{}, std::false_type{});
+        if (kt + 3 == nk) { k_step(std::true_type{}, std::true_type{}, std::true_type{}); ++kt; }
+        if (kt + 2 == nk) { k_step(std::true_type{}, std::false_type{}, std::false_type{}); ++kt; }
+        if (kt + 1 == nk) { k_step(std::false_type{}, std::false_type{}, std::false_type{}); ++kt; }
+    }
 
     // Epilogue.  acc[i][j][4*q+e] = C[row0 + wm*TM*32 + i*32 + (lane&31)]
     //                                [col0 + wn*TN*32 + j*32 + 8*q + 4*(lane>>5) + e]
@@ -399,6 +621,7 @@ int launch_fast(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red,
     else fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, false, OUT>);
     int lds_bytes = 2 * ((a_red ? kRedTileBytes : kOuterTileBytes) + (b_red ? kRedTileBytes : kOuterTileBytes));
     if (OUT == OUT_SAME && lds_bytes < kStageBytes) lds_bytes = kStageBytes;
+    if (!a_red && !b_red && lds_bytes < kRingBytes) lds_bytes = kRingBytes;   // use_ring<false, false>()
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "ms_gmm: hipFuncSetAttribute: %s", hipGetErrorString(e));
     GmmArgs copy = args;
