@@ -25,18 +25,30 @@ namespace ms {
 namespace {
 
 // ---- schedule ------------------------------------------------------------------------
-// One entry per group.  With split_tails the last row tile of a group may be a smaller one (64 or 128
-// rows, the smallest that holds the remainder), so ragged groups do not pay for a whole extra tile; it
-// stays in the group's tile range, next to the full tiles of the same column panel, so the weight panel
-// it reads is being read by its neighbours at the same time.
+// With split_tails the last row tile of a group may be a smaller one (64 or 128 rows, the smallest that
+// holds the remainder), so ragged groups do not pay for a whole extra tile.  part = 0: one entry for the
+// whole group; the small tile stays in the group's tile range, next to the full tiles of the same column
+// panel, so the weight panel it reads is being read by its neighbours at the same time.  part = 1 / 2: the
+// group's full tiles / its small tile as entries of their own (used when the small tiles of all groups are
+// scheduled after all full tiles).
 __device__ __forceinline__ int emit_rows(TileTable *table, int n, int &tiles, GroupEntry e, int tile_rows,
-                                         int num_col_tiles, int split_tails) {
+                                         int num_col_tiles, int split_tails, int part) {
     const int rows = e.row_end - e.row_begin;
     if (rows <= 0) return n;
     e.tile_rows = tile_rows;
     e.num_row_tiles = (rows + tile_rows - 1) / tile_rows;
     const int rem = rows - (e.num_row_tiles - 1) * tile_rows;      // rows of the last tile, 1..tile_rows
     e.tail_rows = !split_tails ? 0 : (rem <= 64 ? 64 : (rem <= 128 ? 128 : 0));
+    if (part == 1 && e.tail_rows != 0) {
+        e.num_row_tiles -= 1;
+        e.row_end = e.row_begin + e.num_row_tiles * tile_rows;
+        e.tail_rows = 0;
+        if (e.num_row_tiles == 0) return n;
+    } else if (part == 2) {
+        if (e.tail_rows == 0) return n;
+        e.row_begin += (e.num_row_tiles - 1) * tile_rows;
+        e.num_row_tiles = 1;
+    }
     e.num_tiles = e.num_row_tiles * num_col_tiles;
     e.share = (e.num_tiles + 7) >> 3;
     e.tile_begin = tiles;
@@ -48,8 +60,9 @@ __device__ __forceinline__ int emit_rows(TileTable *table, int n, int &tiles, Gr
 __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__restrict__ group_list,
                                                            int group_list_type, int group_type, int num_groups,
                                                            int m, int k, int tile_rows, int num_col_tiles,
-                                                           int split_tails, int64_t b_stride_group,
-                                                           int64_t c_stride_group, TileTable *table) {
+                                                           int split_tails, int tails_last_below,
+                                                           int64_t b_stride_group, int64_t c_stride_group,
+                                                           TileTable *table) {
     extern __shared__ int64_t gl[];
     for (int g = threadIdx.x; g < num_groups; g += blockDim.x) gl[g] = group_list[g];
     __syncthreads();
@@ -59,7 +72,24 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
     int64_t prev = 0;
     // Split on the reduction dim: a tile's cost is its group's reduction length, so groups with an
     // above-average length are emitted first (they start early on every XCD), the short ones fill in after.
-    const int passes = group_type == 2 ? 2 : 1;
+    //
+    // Split on rows with small tail tiles: when the launch has only a few rounds of tiles (fewer than
+    // tails_last_below tiles in all), the small tiles of all groups are scheduled after all full tiles, so
+    // that the last, partly filled round is made of the short tiles; with many rounds they stay next to
+    // their group's full tiles, where they find the group's weight panel in L2.
+    bool tails_last = false;
+    if (group_type == 0 && split_tails) {
+        int64_t total = 0, p0 = 0;
+        for (int g = 0; g < num_groups; ++g) {
+            int64_t end = group_list_type == 0 ? gl[g] : p0 + gl[g];
+            end = end < p0 ? p0 : end;
+            end = end > m ? m : end;
+            total += (end - p0 + tile_rows - 1) / tile_rows * num_col_tiles;
+            p0 = end;
+        }
+        tails_last = total < tails_last_below;
+    }
+    const int passes = (group_type == 2 || tails_last) ? 2 : 1;
     const int64_t mean_len = num_groups > 0 ? m / num_groups : 0;
     for (int pass = 0; pass < passes; ++pass) {
         prev = 0;
@@ -68,7 +98,7 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
             end = end < prev ? prev : end;
             end = end > m ? m : end;
             const bool is_long = end - prev >= mean_len;
-            if (passes == 1 || is_long == (pass == 0)) {
+            if (passes == 1 || tails_last || is_long == (pass == 0)) {
                 GroupEntry e{};
                 if (group_type == 0) {
                     e.row_begin = static_cast<int>(prev);
@@ -85,7 +115,7 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
                     e.b_off = 0;
                     e.c_off = g * c_stride_group;
                 }
-                n = emit_rows(table, n, tiles, e, tile_rows, num_col_tiles, split_tails);
+                n = emit_rows(table, n, tiles, e, tile_rows, num_col_tiles, split_tails, tails_last ? pass + 1 : 0);
             }
             prev = end;
         }
@@ -94,7 +124,7 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
         GroupEntry e{};
         e.row_begin = static_cast<int>(prev);
         e.row_end = m;
-        n = emit_rows(table, n, tiles, e, tile_rows, num_col_tiles, split_tails);
+        n = emit_rows(table, n, tiles, e, tile_rows, num_col_tiles, split_tails, 0);
     }
     table->slots_per_xcd = tiles;
     table->num_entries = n;
@@ -395,8 +425,24 @@ __global__ __launch_bounds__(256) void gmm32_kernel(const GmmArgs p) {
 }
 
 // ---- host -------------------------------------------------------------------------------
+// A launch with fewer than this many rounds of tiles (tiles / compute units) schedules its small tail tiles last.
+constexpr int kTailsLastRounds = 4;
+
+// Compute units of the current device (cached per device ordinal; 256 if the query fails).
+int current_device_cus() {
+    static int cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 size_t table_bytes(int64_t num_groups) {
-    return sizeof(TileTable) + static_cast<size_t>(num_groups + 2) * sizeof(GroupEntry);
+    return sizeof(TileTable) + static_cast<size_t>(2 * num_groups + 2) * sizeof(GroupEntry);   // full + tail entries
 }
 
 template <int DT, int OUT>
@@ -482,11 +528,12 @@ extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int
 
     TileTable *table = static_cast<TileTable *>(workspace);
     const int64_t c_stride_group = k * y_stride_row;
+    const int num_cus = current_device_cus();
     auto schedule = [&](int split_tails) -> int {
         hipLaunchKernelGGL(gmm_schedule_kernel, dim3(1), dim3(256), static_cast<size_t>(num_groups) * sizeof(int64_t),
                            stream, group_list, group_list_type, group_type, static_cast<int>(num_groups),
                            static_cast<int>(m), static_cast<int>(k), tile_rows, static_cast<int>(num_col_tiles),
-                           split_tails, w_stride_group, c_stride_group, table);
+                           split_tails, kTailsLastRounds * num_cus, w_stride_group, c_stride_group, table);
         MS_CHECK_LAUNCH("gmm_schedule_kernel");
         return MS_OK;
     };
@@ -503,7 +550,7 @@ extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int
     args.c_stride_row = y_stride_row;
     args.cols = static_cast<int>(n);
     args.num_col_tiles = static_cast<int>(num_col_tiles);
-    const unsigned grid = static_cast<unsigned>((ceil_div(tiles_bound, 8) + num_groups + 2) * 8);
+    const unsigned grid = static_cast<unsigned>((ceil_div(tiles_bound, 8) + 2 * num_groups + 2) * 8);
 
     if (is32) {
         if (int rc = schedule(0)) return rc;
