@@ -116,6 +116,57 @@ def cpu_baseline(cfg, budget_s=15.0):
                       f"({dt:.1f} s) with torch {torch.__version__} on {threads} threads"}
 
 
+def measure_routing_map_mode(cfg, device, x, idx, p, iters=20, warmup=5):
+    """The routing-map (mask) form of permute / unpermute on the same workload: event-timed averages of the
+    forward and of forward+backward, with the algorithmic bytes of the row movement.  Not part of `value`."""
+    from mindspeed_amd.ops import moe_permute_mask_map as M
+
+    T, H, E, K = cfg["T"], cfg["H"], cfg["E"], cfg["K"]
+    rmap = torch.zeros(T, E, dtype=torch.bool, device=device)
+    rmap.scatter_(1, idx, True)
+    rows = int(rmap.sum().item())
+    probs = torch.zeros(T, E, dtype=torch.float32, device=device).scatter_(1, idx, p.float())
+    elem = x.element_size()
+    xg = x.detach().clone().requires_grad_(True)
+    pg = probs.clone().requires_grad_(True)
+    perm, _, sidx = M.permute(xg, rmap, pg, num_out_tokens=rows, fused=True)
+    rg = perm.detach().clone().requires_grad_(True)
+    g_rows, g_out = torch.randn_like(perm), torch.randn_like(x)
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    def permute_fb():
+        out, _, _ = M.permute(xg, rmap, pg, num_out_tokens=rows, fused=True)
+        torch.autograd.grad(out, xg, g_rows)
+
+    def unpermute_fb():
+        out = M.unpermute(rg, sidx, x.shape, probs=pg, routing_map=rmap, fused=True)
+        torch.autograd.grad(out, (rg, pg), g_out)
+
+    t_pf = timed(lambda: M.permute(x, rmap, probs, num_out_tokens=rows, fused=True))
+    t_pfb = timed(permute_fb)
+    t_uf = timed(lambda: M.unpermute(perm.detach(), sidx, x.shape, probs=probs, routing_map=rmap, fused=True))
+    t_ufb = timed(unpermute_fb)
+    move = (T + rows) * H * elem       # rows read once + rows written once, either direction
+    return {
+        "note": "routing-map (mask) form on the same routing; every call re-sorts the [T, E] mask on the device",
+        "rows": rows,
+        "permute_fwd": {"avg_ms": round(t_pf, 5), "gbs": round(move / t_pf / 1e6, 1)},
+        "permute_fwd_bwd": {"avg_ms": round(t_pfb, 5), "gbs": round(2 * move / t_pfb / 1e6, 1)},
+        "unpermute_fwd": {"avg_ms": round(t_uf, 5), "gbs": round(move / t_uf / 1e6, 1)},
+        "unpermute_fwd_bwd": {"avg_ms": round(t_ufb, 5), "gbs": round((move + (T + 2 * rows) * H * elem) / t_ufb / 1e6, 1)},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -224,6 +275,7 @@ def main():
             _lib.check(lib.ms_copy_bytes(_lib.stream_ptr(device), _lib.ptr(src), _lib.ptr(dst), n), "ms_copy_bytes")
         torch.cuda.synchronize()
         result["copy_calibration_bytes"] = n
+    result["routing_map_mode"] = measure_routing_map_mode(cfg, device, x.detach(), idx, p.detach())
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(result))

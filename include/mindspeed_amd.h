@@ -111,6 +111,51 @@ int ms_moe_token_unpermute_grad(ms_stream_t stream, const void *permuted_tokens,
                                 void *grad_permuted_tokens, void *grad_probs);
 
 /* ------------------------------------------------------------------------
+ * Routing-map (mask) mode of permute / unpermute — stands in for
+ * torch_npu.npu_moe_token_permute_with_routing_map[_grad] and
+ * torch_npu._npu_moe_token_unpermute_with_routing_map[_grad] as called from
+ * mindspeed/te/pytorch/permutation.py:23-24,52-60,84-86,118-142 (Python surface
+ * mindspeed/core/fusions/fused_moe_permute.py:50-85).
+ *
+ * routing_map [num_tokens, num_experts] bytes (torch.bool).  Flat entry
+ * i = t*num_experts + e.  Without drop-and-pad the set entries are laid out
+ * expert-major, token-ascending:
+ *   permuted_tokens [num_out_tokens, hidden]     row r = tokens[sorted_flat[r] / num_experts]
+ *   row_id_map  int32 [num_tokens*num_experts]   output row of flat entry i; unset entries and
+ *                                                rows >= num_out_tokens hold 0x7fffffff (dropped)
+ *   sorted_flat int32 [num_out_tokens]           flat entry of row r (-1 for a row nothing maps to,
+ *                                                which only happens when num_out_tokens exceeds the
+ *                                                number of set entries; such rows are not written)
+ *   tokens_per_expert int64 [num_experts]        optional: set entries per expert
+ * With drop_and_pad != 0, num_out_tokens = num_experts * capacity and expert e owns rows
+ * [e*capacity, (e+1)*capacity): its routed tokens in ascending order, then (as padding) its
+ * non-routed tokens in ascending order, cut at capacity — the selection
+ * routing_map.T.argsort(descending, stable)[:, :capacity] makes; tokens_per_expert = capacity.
+ * tokens / permuted_tokens may be NULL to compute the maps only (unpermute needs them again).
+ * The row maps plug into ms_moe_token_permute_grad / ms_moe_token_unpermute[_grad] with
+ * topk = num_experts.
+ *
+ * ms_moe_routing_map_probs:      permuted_probs[r] = probs.flat[sorted_flat[r]] (0 for r unmapped),
+ *                                sorted_token_ids[r] = sorted_flat[r] / num_experts (int64, the
+ *                                sorted_indices the Python surface returns); either output may be NULL.
+ * ms_moe_routing_map_probs_grad: grad_probs.flat[i] = grad_permuted_probs[row_id_map[i]], 0 for
+ *                                dropped entries.
+ * ---------------------------------------------------------------------- */
+int ms_moe_routing_map_workspace_size(int64_t num_tokens, int64_t num_experts, int drop_and_pad,
+                                      size_t *bytes);
+int ms_moe_routing_map_permute(ms_stream_t stream, const void *tokens, const void *routing_map,
+                               int64_t num_tokens, int64_t num_experts, int64_t hidden, int dtype,
+                               int64_t num_out_tokens, int drop_and_pad, void *permuted_tokens,
+                               int32_t *row_id_map, int32_t *sorted_flat, int64_t *tokens_per_expert,
+                               void *workspace, size_t workspace_bytes);
+int ms_moe_routing_map_probs(ms_stream_t stream, const int32_t *sorted_flat, int64_t num_out_tokens,
+                             int64_t num_experts, const void *probs, int dtype, void *permuted_probs,
+                             int64_t *sorted_token_ids);
+int ms_moe_routing_map_probs_grad(ms_stream_t stream, const int32_t *row_id_map, int64_t num_entries,
+                                  const void *grad_permuted_probs, int dtype, int64_t num_out_tokens,
+                                  void *grad_probs);
+
+/* ------------------------------------------------------------------------
  * Grouped matmul — stands in for aclnnGroupedMatmulV2 / V4 as called from
  * mindspeed/ops/csrc/cann/gmm.cpp:77-167 (Python surface
  * mindspeed/ops/gmm.py:164-175), including the backward recipes of

@@ -534,6 +534,73 @@ __global__ void copy_tail_kernel(const unsigned char *src, unsigned char *dst, s
     if (i < end) dst[i] = src[i];
 }
 
+// ---- routing-map (mask) mode ----------------------------------------------------------
+// The [T, E] boolean routing map is sorted with the same counting sort as the index form: flat position
+// i = t*E + e gets the key e when the entry is set and the extra last key E when it is not, so the set
+// entries come out expert-major, token-ascending (rows 0 .. nnz-1) and the unset ones after them.  In
+// drop-and-pad mode the key is 2*e + (entry unset): every expert's block then holds all T tokens, routed
+// ones first, and the first `capacity` of each block are kept, which is what
+// argsort(descending, stable)[:, :capacity] on the transposed int8 map selects.
+__global__ __launch_bounds__(256) void routing_map_keys_kernel(const unsigned char *__restrict__ map, int n, int E,
+                                                               int pad, int32_t *__restrict__ keys,
+                                                               int32_t *__restrict__ sorted_flat, int num_rows) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const int e = i % E;
+        const bool set = map[i] != 0;
+        keys[i] = pad ? 2 * e + (set ? 0 : 1) : (set ? e : E);
+    }
+    if (i < num_rows) sorted_flat[i] = -1;   // rows nobody maps to stay marked
+}
+
+// rank[i] (position of flat entry i in the sorted order) -> output row, in place; the inverse list
+// sorted_flat[row] = i; rows per expert.  counts: per-key totals of the sort (E+1 keys, or 2E in pad mode).
+__global__ __launch_bounds__(256) void routing_map_rows_kernel(const int32_t *__restrict__ keys, int n, int T, int E,
+                                                               int capacity, int num_rows,
+                                                               int32_t *__restrict__ row_id_map,
+                                                               int32_t *__restrict__ sorted_flat,
+                                                               const int64_t *__restrict__ counts,
+                                                               int64_t *__restrict__ tokens_per_expert) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (tokens_per_expert != nullptr && i < E) tokens_per_expert[i] = capacity > 0 ? capacity : counts[i];
+    if (i >= n) return;
+    const int rank = row_id_map[i];
+    int row = -1;
+    if (capacity > 0) {
+        const int e = rank / T, j = rank - e * T;
+        if (j < capacity) row = e * capacity + j;
+    } else if (keys[i] < E) {
+        row = rank;
+    }
+    if (static_cast<unsigned>(row) >= static_cast<unsigned>(num_rows)) row = -1;
+    row_id_map[i] = row < 0 ? 0x7fffffff : row;   // dropped: an id no row count reaches
+    if (row >= 0) sorted_flat[row] = i;
+}
+
+// permuted_probs[r] = probs.flat[sorted_flat[r]], sorted_token_ids[r] = sorted_flat[r] / E (0 for unmapped rows)
+template <typename S>
+__global__ __launch_bounds__(256) void routing_map_probs_kernel(const int32_t *__restrict__ sorted_flat, int num_rows,
+                                                                int E, const S *__restrict__ probs,
+                                                                S *__restrict__ permuted_probs,
+                                                                int64_t *__restrict__ sorted_token_ids) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= num_rows) return;
+    const int i = sorted_flat[r];
+    if (permuted_probs != nullptr) permuted_probs[r] = i >= 0 ? probs[i] : S(0);
+    if (sorted_token_ids != nullptr) sorted_token_ids[r] = i >= 0 ? i / E : 0;
+}
+
+// grad_probs.flat[i] = grad_permuted_probs[row_id_map[i]] for mapped entries, 0 otherwise
+template <typename S>
+__global__ __launch_bounds__(256) void routing_map_probs_grad_kernel(const int32_t *__restrict__ row_id_map, int n,
+                                                                     const S *__restrict__ grad_permuted_probs,
+                                                                     int num_rows, S *__restrict__ grad_probs) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int r = row_id_map[i];
+    grad_probs[i] = static_cast<unsigned>(r) < static_cast<unsigned>(num_rows) ? grad_permuted_probs[r] : S(0);
+}
+
 // ---- host helpers -------------------------------------------------------------------
 struct SortPlan {
     int n, nbins, nbits, seg, nseg;
@@ -765,6 +832,136 @@ extern "C" int ms_moe_token_unpermute_grad(ms_stream_t stream_, const void *perm
         case MS_FP16: return launch_unpermute_grad<FP16>(stream, permuted, grad_out, row_id_map, probs, grad_permuted, grad_probs, T, k, H, num_rows);
         default: return launch_unpermute_grad<FP32>(stream, permuted, grad_out, row_id_map, probs, grad_permuted, grad_probs, T, k, H, num_rows);
     }
+}
+
+// ---- routing-map mode entry points ------------------------------------------------------
+namespace {
+struct RoutingPlan {
+    int64_t n;          // T * E flat entries
+    int nkeys;          // E + 1, or 2 * E in drop-and-pad mode
+    ms::SortPlan sort;
+    size_t keys_off, counts_off, sort_off, total;
+};
+RoutingPlan make_routing_plan(int64_t T, int64_t E, int pad) {
+    RoutingPlan r{};
+    r.n = T * E;
+    r.nkeys = static_cast<int>(pad ? 2 * E : E + 1);
+    r.sort = ms::make_sort_plan(r.n, r.nkeys);
+    auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
+    r.keys_off = 0;
+    r.counts_off = up(static_cast<size_t>(r.n) * sizeof(int32_t));
+    r.sort_off = r.counts_off + up(static_cast<size_t>(r.nkeys) * sizeof(int64_t));
+    r.total = r.sort_off + up(r.sort.small ? 0 : static_cast<size_t>(r.sort.nseg) * r.sort.nbins * sizeof(int));
+    return r;
+}
+int check_routing(const char *fn, int64_t T, int64_t E, int pad) {
+    MS_REQUIRE(T >= 0 && E >= 1, MS_ERR_INVALID_ARGUMENT, "%s: need num_tokens >= 0, num_experts >= 1", fn);
+    MS_REQUIRE((pad ? 2 * E : E + 1) <= MS_MAX_EXPERTS, MS_ERR_UNSUPPORTED, "%s: num_experts %lld too large (limit %d%s)",
+               fn, (long long)E, pad ? MS_MAX_EXPERTS / 2 : MS_MAX_EXPERTS - 1, pad ? " in drop-and-pad mode" : "");
+    MS_REQUIRE(T * E < (1ll << 31) - 64, MS_ERR_UNSUPPORTED, "%s: num_tokens*num_experts must fit int32", fn);
+    return MS_OK;
+}
+}  // namespace
+
+extern "C" int ms_moe_routing_map_workspace_size(int64_t T, int64_t E, int drop_and_pad, size_t *bytes) {
+    MS_REQUIRE(bytes != nullptr, MS_ERR_INVALID_ARGUMENT, "ms_moe_routing_map_workspace_size: bytes is NULL");
+    if (int rc = check_routing("ms_moe_routing_map_workspace_size", T, E, drop_and_pad)) return rc;
+    *bytes = make_routing_plan(T, E, drop_and_pad).total;
+    return MS_OK;
+}
+
+extern "C" int ms_moe_routing_map_permute(ms_stream_t stream_, const void *tokens, const void *routing_map, int64_t T,
+                                          int64_t E, int64_t H, int dtype, int64_t num_rows, int drop_and_pad,
+                                          void *permuted, int32_t *row_id_map, int32_t *sorted_flat,
+                                          int64_t *tokens_per_expert, void *workspace, size_t workspace_bytes) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char *fn = "ms_moe_routing_map_permute";
+    if (int rc = check_routing(fn, T, E, drop_and_pad)) return rc;
+    MS_REQUIRE(num_rows >= 0 && num_rows <= T * E, MS_ERR_INVALID_ARGUMENT, "%s: num_out_tokens %lld outside [0, %lld]", fn,
+               (long long)num_rows, (long long)(T * E));
+    MS_REQUIRE(!drop_and_pad || (num_rows % E == 0 && num_rows / E <= T), MS_ERR_INVALID_ARGUMENT,
+               "%s: drop-and-pad needs num_out_tokens = num_experts * capacity with capacity <= num_tokens (got %lld)", fn,
+               (long long)num_rows);
+    if (tokens != nullptr)
+        if (int rc = check_common(fn, T, E, H, dtype)) return rc;
+    if (T == 0) return MS_OK;
+    MS_REQUIRE(routing_map && row_id_map && sorted_flat, MS_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", fn);
+    MS_REQUIRE(tokens == nullptr || permuted != nullptr || num_rows == 0, MS_ERR_INVALID_ARGUMENT, "%s: permuted is NULL", fn);
+    const RoutingPlan r = make_routing_plan(T, E, drop_and_pad);
+    MS_REQUIRE(workspace != nullptr && workspace_bytes >= r.total, MS_ERR_WORKSPACE_TOO_SMALL, "%s: workspace %zu < %zu bytes",
+               fn, workspace_bytes, r.total);
+    MS_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7u) == 0, MS_ERR_INVALID_ARGUMENT, "%s: workspace must be 8-byte aligned", fn);
+    char *ws = static_cast<char *>(workspace);
+    int32_t *keys = reinterpret_cast<int32_t *>(ws + r.keys_off);
+    int64_t *counts = reinterpret_cast<int64_t *>(ws + r.counts_off);
+    const int n = static_cast<int>(r.n);
+    const int capacity = drop_and_pad ? static_cast<int>(num_rows / E) : 0;
+    const int64_t cover = r.n > num_rows ? r.n : num_rows;
+    hipLaunchKernelGGL(routing_map_keys_kernel, dim3(static_cast<unsigned>(ceil_div(cover, 256))), dim3(256), 0, stream,
+                       static_cast<const unsigned char *>(routing_map), n, static_cast<int>(E), drop_and_pad ? 1 : 0, keys,
+                       sorted_flat, static_cast<int>(num_rows));
+    MS_CHECK_LAUNCH("routing_map_keys_kernel");
+    if (int rc = launch_sort(stream, r.sort, keys, 0, row_id_map, nullptr, counts, r.nkeys, ws + r.sort_off)) return rc;
+    hipLaunchKernelGGL(routing_map_rows_kernel, dim3(static_cast<unsigned>(ceil_div(r.n, 256))), dim3(256), 0, stream, keys, n,
+                       static_cast<int>(T), static_cast<int>(E), capacity, static_cast<int>(num_rows), row_id_map, sorted_flat,
+                       counts, tokens_per_expert);
+    MS_CHECK_LAUNCH("routing_map_rows_kernel");
+    if (tokens == nullptr || num_rows == 0) return MS_OK;
+    const int64_t row_bytes = H * dtype_size(dtype);
+    if (row_bytes % 16 == 0 && aligned16(tokens) && aligned16(permuted))
+        return launch_permute_rows<v16>(stream, tokens, permuted, row_id_map, T, E, row_bytes, num_rows);
+    if (dtype == MS_FP32) return launch_permute_rows<uint32_t>(stream, tokens, permuted, row_id_map, T, E, row_bytes, num_rows);
+    return launch_permute_rows<uint16_t>(stream, tokens, permuted, row_id_map, T, E, row_bytes, num_rows);
+}
+
+extern "C" int ms_moe_routing_map_probs(ms_stream_t stream_, const int32_t *sorted_flat, int64_t num_rows, int64_t E,
+                                        const void *probs, int dtype, void *permuted_probs, int64_t *sorted_token_ids) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char *fn = "ms_moe_routing_map_probs";
+    MS_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31) && E >= 1, MS_ERR_INVALID_ARGUMENT, "%s: bad sizes", fn);
+    MS_REQUIRE((probs == nullptr) == (permuted_probs == nullptr), MS_ERR_INVALID_ARGUMENT,
+               "%s: probs and permuted_probs must be given together", fn);
+    MS_REQUIRE(probs == nullptr || dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED,
+               "%s: dtype %d is not one of bf16/fp16/fp32", fn, dtype);
+    if (num_rows == 0) return MS_OK;
+    MS_REQUIRE(sorted_flat != nullptr, MS_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", fn);
+    const dim3 grid(static_cast<unsigned>(ceil_div(num_rows, 256)));
+    // a probability is only moved, never computed with: 2-byte types share one instantiation
+    if (probs != nullptr && dtype == MS_FP32)
+        hipLaunchKernelGGL(routing_map_probs_kernel<uint32_t>, grid, dim3(256), 0, stream, sorted_flat, static_cast<int>(num_rows),
+                           static_cast<int>(E), static_cast<const uint32_t *>(probs), static_cast<uint32_t *>(permuted_probs),
+                           sorted_token_ids);
+    else
+        hipLaunchKernelGGL(routing_map_probs_kernel<uint16_t>, grid, dim3(256), 0, stream, sorted_flat, static_cast<int>(num_rows),
+                           static_cast<int>(E), static_cast<const uint16_t *>(probs), static_cast<uint16_t *>(permuted_probs),
+                           sorted_token_ids);
+    MS_CHECK_LAUNCH("routing_map_probs_kernel");
+    return MS_OK;
+}
+
+extern "C" int ms_moe_routing_map_probs_grad(ms_stream_t stream_, const int32_t *row_id_map, int64_t num_entries,
+                                             const void *grad_permuted_probs, int dtype, int64_t num_rows,
+                                             void *grad_probs) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char *fn = "ms_moe_routing_map_probs_grad";
+    MS_REQUIRE(num_entries >= 0 && num_entries < (1ll << 31) && num_rows >= 0 && num_rows < (1ll << 31),
+               MS_ERR_INVALID_ARGUMENT, "%s: bad sizes", fn);
+    MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED,
+               "%s: dtype %d is not one of bf16/fp16/fp32", fn, dtype);
+    if (num_entries == 0) return MS_OK;
+    MS_REQUIRE(row_id_map && grad_probs && (grad_permuted_probs || num_rows == 0), MS_ERR_INVALID_ARGUMENT,
+               "%s: NULL tensor pointer", fn);
+    const dim3 grid(static_cast<unsigned>(ceil_div(num_entries, 256)));
+    if (dtype == MS_FP32)
+        hipLaunchKernelGGL(routing_map_probs_grad_kernel<uint32_t>, grid, dim3(256), 0, stream, row_id_map,
+                           static_cast<int>(num_entries), static_cast<const uint32_t *>(grad_permuted_probs),
+                           static_cast<int>(num_rows), static_cast<uint32_t *>(grad_probs));
+    else
+        hipLaunchKernelGGL(routing_map_probs_grad_kernel<uint16_t>, grid, dim3(256), 0, stream, row_id_map,
+                           static_cast<int>(num_entries), static_cast<const uint16_t *>(grad_permuted_probs),
+                           static_cast<int>(num_rows), static_cast<uint16_t *>(grad_probs));
+    MS_CHECK_LAUNCH("routing_map_probs_grad_kernel");
+    return MS_OK;
 }
 
 extern "C" int ms_copy_bytes(ms_stream_t stream_, const void *src, void *dst, size_t bytes) {

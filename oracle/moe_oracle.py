@@ -32,6 +32,17 @@ groupmatmul_add_fp32          pinned: equals ``out + dw`` (the reference
                               test's own identity).
 swiglu                        pinned: closed form ``x*sigmoid(x)*u`` in fp64.
 sort_chunks_by_idxs           pinned: brute-force row map.
+permute_routing_map /         pinned: brute-force Python loops over (expert, token)
+unpermute_routing_map         pairs incl. drop-and-pad, equality with the index
+                              form (permute / unpermute above) on maps built from
+                              top-k indices, the in-tree formulas
+                              (token_dispatcher.py:451-453,
+                              unpermute_without_activation.py:44-62); backward =
+                              autograd of these differentiable restatements.
+                              The algorithm itself is Megatron-LM core_r0.12
+                              ``moe_utils.permute/unpermute`` (a dependency that
+                              is not vendored in the reference tree), restated
+                              from its published source.
 fused-op output conventions   PARITY UNPINNED: what the closed vendor kernels
   (second output of           ``aclnnMoeTokenPermute`` / ``aclnnGroupedMatmul``
   npu_moe_token_permute,      really return for dropped rows, rows past the
@@ -48,6 +59,7 @@ __all__ = [
     "permute_backward", "unpermute_backward", "grouped_matmul", "gmm_split",
     "gmm", "gmm_backward", "groupmatmul_add_fp32", "swiglu", "swiglu_backward",
     "sort_chunks_by_idxs", "experts_computation", "moe_layer", "route_topk",
+    "permute_routing_map", "unpermute_routing_map",
 ]
 
 
@@ -382,3 +394,64 @@ def route_topk(logits, topk):
     p, idx = torch.topk(probs_full, topk, dim=-1)
     p = p / p.sum(dim=-1, keepdim=True)
     return p, idx
+
+
+# --------------------------------------------------------------------------
+# routing-map (mask) mode
+# --------------------------------------------------------------------------
+def permute_routing_map(tokens, routing_map, probs=None, num_out_tokens=None, drop_and_pad=False):
+    """Megatron-LM core_r0.12 ``moe_utils.permute`` (the function the reference's
+    mindspeed/core/fusions/fused_moe_permute.py:65-66 falls back to and that the vendor op behind
+    mindspeed/te/pytorch/permutation.py:23-24 replaces).
+
+    ``routing_map`` ``[T, E]`` bool, ``probs`` ``[T, E]``.  Returns
+    ``(permuted_tokens, permuted_probs, sorted_indices)`` with ``sorted_indices`` the token id of every
+    output row, rows expert-major and token-ascending.  ``drop_and_pad``: ``capacity = num_out_tokens // E``
+    rows per expert, chosen by a stable descending argsort of the transposed map (routed tokens first,
+    non-routed tokens as padding)."""
+    num_tokens, _ = tokens.shape
+    num_experts = routing_map.shape[1]
+    permuted_probs = None
+    if drop_and_pad and num_out_tokens is not None:
+        capacity = num_out_tokens // num_experts
+        rm = routing_map.to(torch.int8).T.contiguous()
+        sorted_indices = rm.argsort(dim=-1, descending=True, stable=True)[:, :capacity].contiguous().view(-1)
+        if probs is not None:
+            probs_t = probs.T.contiguous().view(-1)
+            dim0 = torch.arange(num_experts).unsqueeze(-1)
+            flat = (dim0 * num_tokens + sorted_indices.view(num_experts, capacity)).view(-1)
+            permuted_probs = probs_t.index_select(0, flat)
+    else:
+        rm = routing_map.bool().T.contiguous()
+        token_indices = torch.arange(num_tokens).unsqueeze(0).expand(num_experts, -1)
+        sorted_indices = token_indices.masked_select(rm)
+        if probs is not None:
+            # same expression as mindspeed/core/transformer/moe/moe_feature/overlap/token_dispatcher.py:451-453
+            permuted_probs = probs.T.contiguous().masked_select(rm)
+    permuted = tokens.index_select(0, sorted_indices)
+    return permuted, permuted_probs, sorted_indices
+
+
+def unpermute_routing_map(permuted_tokens, sorted_indices, restore_shape, probs=None, routing_map=None,
+                          drop_and_pad=False):
+    """Megatron-LM core_r0.12 ``moe_utils.unpermute``; its non-padded branch is restated in-tree at
+    mindspeed/core/transformer/moe/unpermute_without_activation.py:44-62: rows are scaled by their
+    permuted probability and scatter-added into ``zeros(restore_shape)`` by token id; the product and
+    the sum are in the promoted dtype, the result is cast back to the input dtype."""
+    _, hidden = restore_shape
+    input_dtype = permuted_tokens.dtype
+    if probs is not None:
+        if drop_and_pad:
+            num_experts = routing_map.size(1)
+            capacity = sorted_indices.size(0) // num_experts
+            num_unpermuted = probs.size(0)
+            probs_t = probs.T.contiguous().view(-1)
+            dim0 = torch.arange(num_experts).unsqueeze(-1)
+            flat = (dim0 * num_unpermuted + sorted_indices.view(num_experts, capacity)).view(-1)
+            permuted_probs = probs_t.index_select(0, flat)
+        else:
+            permuted_probs = probs.T.contiguous().masked_select(routing_map.T.contiguous())
+        permuted_tokens = permuted_tokens * permuted_probs.unsqueeze(-1)
+    out = torch.zeros(restore_shape, dtype=permuted_tokens.dtype)
+    out = out.scatter_add(0, sorted_indices.unsqueeze(1).expand(-1, hidden), permuted_tokens)
+    return out.to(input_dtype)

@@ -1,0 +1,201 @@
+"""GPU parity: routing-map (mask) mode of permute / unpermute against the CPU oracle, through the Python
+surface that calls the C ABI.  Index outputs, permuted rows and permuted probabilities are compared
+bit-exactly; weighted sums within rel-L2 1e-2 (bf16, fp16) and 1e-5 (fp32)."""
+import pytest
+import torch
+
+from conftest import rel_l2
+from oracle import moe_oracle as O
+
+from mindspeed_amd.ops import moe_permute_mask_map as M
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.bfloat16: 1e-2, torch.float16: 1e-2, torch.float32: 1e-5}
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def make_map(T, E, k, seed, never=()):
+    """Top-k style mask and probabilities; experts listed in ``never`` are never chosen."""
+    gen = torch.Generator().manual_seed(seed)
+    scores = torch.rand(T, E, generator=gen)
+    for e in never:
+        scores[:, e] = -1.0
+    idx = scores.topk(k, dim=1).indices
+    rmap = torch.zeros(T, E, dtype=torch.bool)
+    rmap.scatter_(1, idx, True)
+    probs = torch.where(rmap, torch.rand(T, E, generator=gen) + 0.1, torch.zeros(T, E))
+    return rmap, probs
+
+
+CASES = [
+    # T, E, k, H, dtype, probs dtype, never-chosen experts
+    (1, 1, 1, 8, torch.bfloat16, torch.float32, ()),
+    (9, 4, 2, 16, torch.float32, torch.float32, ()),
+    (64, 8, 2, 128, torch.bfloat16, torch.float32, (3,)),
+    (300, 8, 2, 264, torch.float32, torch.float32, (0, 7)),
+    (257, 5, 3, 70, torch.float16, torch.float16, ()),            # odd hidden: element path
+    (512, 64, 8, 96, torch.bfloat16, torch.bfloat16, ()),         # T*E = 32768: multi-block sort
+    (4096, 8, 2, 512, torch.bfloat16, torch.float32, ()),         # Mixtral routing at reduced hidden
+    (2000, 130, 4, 32, torch.bfloat16, torch.float32, (129,)),    # > 64 experts, ragged
+]
+
+
+@pytest.mark.parametrize("T,E,k,H,dtype,pdt,never", CASES)
+def test_permute_mask_map_forward_backward(T, E, k, H, dtype, pdt, never, device):
+    say("routing-map permute case", T, E, k, H, dtype, pdt, never)
+    rmap, probs = make_map(T, E, k, T * 7 + E, never)
+    probs = probs.to(pdt)
+    gen = torch.Generator().manual_seed(T + 13)
+    tokens = torch.randn(T, H, generator=gen).to(dtype)
+    exp_perm, exp_pp, exp_idx = O.permute_routing_map(tokens, rmap, probs)
+
+    tok_d = tokens.to(device).requires_grad_(True)
+    probs_d = probs.to(device).requires_grad_(True)
+    for num_out in (None, exp_perm.size(0)):
+        perm, pp, sidx = M.permute(tok_d, rmap.to(device), probs_d, num_out_tokens=num_out, fused=True)
+        torch.cuda.synchronize()
+        assert sidx.dtype == torch.int64 and torch.equal(sidx.cpu(), exp_idx)
+        assert torch.equal(perm.detach().cpu(), exp_perm)
+        assert torch.equal(pp.detach().cpu(), exp_pp)
+
+    # backward: random cotangents for both differentiable outputs
+    g_rows = torch.randn(exp_perm.shape, generator=gen).to(dtype)
+    g_pp = torch.randn(exp_pp.shape, generator=gen).to(pdt)
+    (perm * g_rows.to(device)).sum().backward(retain_graph=True)
+    act_grad = tok_d.grad.clone()
+    tok_d.grad = None
+    (pp * g_pp.to(device)).sum().backward()
+    torch.cuda.synchronize()
+    t64 = tokens.double().requires_grad_(True)
+    p64 = probs.double().requires_grad_(True)
+    o_perm, o_pp, _ = O.permute_routing_map(t64, rmap, p64)
+    (o_perm * g_rows.double()).sum().backward(retain_graph=True)
+    (o_pp * g_pp.double()).sum().backward()
+    assert rel_l2(act_grad, t64.grad) <= TOL[dtype]
+    assert torch.equal(probs_d.grad.cpu().double(), p64.grad.to(pdt).double())   # a pure scatter of g_pp
+
+
+@pytest.mark.parametrize("T,E,k,H,dtype,pdt,never", CASES)
+@pytest.mark.parametrize("with_probs", [True, False])
+def test_unpermute_mask_map_forward_backward(T, E, k, H, dtype, pdt, never, with_probs, device):
+    say("routing-map unpermute case", T, E, k, H, dtype, pdt, never, with_probs)
+    rmap, probs = make_map(T, E, k, T * 5 + E + 1, never)
+    probs = probs.to(pdt)
+    gen = torch.Generator().manual_seed(T + 29)
+    tokens = torch.randn(T, H, generator=gen).to(dtype)
+    _, _, sidx = O.permute_routing_map(tokens, rmap)
+    rows = torch.randn(sidx.numel(), H, generator=gen).to(dtype)
+    g_out = torch.randn(T, H, generator=gen).to(dtype)
+
+    rows_d = rows.to(device).requires_grad_(True)
+    probs_d = probs.to(device).requires_grad_(True) if with_probs else None
+    out = M.unpermute(rows_d, sidx.to(device), tokens.shape, probs=probs_d, routing_map=rmap.to(device), fused=True)
+    out.backward(g_out.to(device))
+    torch.cuda.synchronize()
+
+    r64 = rows.double().requires_grad_(True)
+    p64 = probs.double().requires_grad_(True) if with_probs else None
+    exp = O.unpermute_routing_map(r64, sidx, tokens.shape, p64, rmap)
+    exp.backward(g_out.double())
+    assert out.dtype == dtype
+    assert rel_l2(out, exp) <= TOL[dtype]
+    assert rel_l2(rows_d.grad, r64.grad) <= TOL[dtype]
+    if with_probs:
+        mask = rmap.double()
+        assert rel_l2(probs_d.grad.cpu().double() * mask, p64.grad * mask) <= TOL[dtype]
+        assert torch.count_nonzero(probs_d.grad.cpu().double() * (1 - mask)) == 0   # unset entries get no gradient
+
+
+PAD_CASES = [
+    # T, E, k, capacity, H, dtype
+    (9, 4, 2, 3, 16, torch.float32),
+    (64, 8, 2, 10, 128, torch.bfloat16),     # some experts over capacity (drop), some under (pad)
+    (100, 5, 1, 100, 40, torch.float32),     # capacity = T: every token appears for every expert
+    (3000, 8, 2, 700, 64, torch.bfloat16),   # T*E = 24000: multi-block sort, 16 keys
+    (500, 16, 4, 1, 8, torch.float16),
+]
+
+
+@pytest.mark.parametrize("T,E,k,cap,H,dtype", PAD_CASES)
+def test_drop_and_pad(T, E, k, cap, H, dtype, device):
+    say("routing-map drop_and_pad case", T, E, k, cap, H, dtype)
+    rmap, probs = make_map(T, E, k, T * 3 + cap)
+    gen = torch.Generator().manual_seed(T + 41)
+    tokens = torch.randn(T, H, generator=gen).to(dtype)
+    n = E * cap
+    exp_perm, exp_pp, exp_idx = O.permute_routing_map(tokens, rmap, probs, num_out_tokens=n, drop_and_pad=True)
+    tok_d = tokens.to(device).requires_grad_(True)
+    probs_d = probs.to(device).requires_grad_(True)
+    perm, pp, sidx = M.permute(tok_d, rmap.to(device), probs_d, num_out_tokens=n, fused=True, drop_and_pad=True)
+    torch.cuda.synchronize()
+    assert torch.equal(sidx.cpu(), exp_idx)
+    assert torch.equal(perm.detach().cpu(), exp_perm)
+    assert torch.equal(pp.detach().cpu(), exp_pp)
+
+    g_rows = torch.randn(exp_perm.shape, generator=gen).to(dtype)
+    (perm * g_rows.to(device)).sum().backward()
+    t64 = tokens.double().requires_grad_(True)
+    o_perm, _, _ = O.permute_routing_map(t64, rmap, probs.double(), num_out_tokens=n, drop_and_pad=True)
+    (o_perm * g_rows.double()).sum().backward()
+    assert rel_l2(tok_d.grad, t64.grad) <= TOL[dtype]
+
+    # unpermute in the same mode
+    rows = torch.randn(n, H, generator=gen).to(dtype)
+    g_out = torch.randn(T, H, generator=gen).to(dtype)
+    rows_d = rows.to(device).requires_grad_(True)
+    probs_u = probs.to(device).requires_grad_(True)
+    out = M.unpermute(rows_d, sidx, tokens.shape, probs=probs_u, routing_map=rmap.to(device), fused=True,
+                      drop_and_pad=True)
+    out.backward(g_out.to(device))
+    torch.cuda.synchronize()
+    r64 = rows.double().requires_grad_(True)
+    p64 = probs.double().requires_grad_(True)
+    exp = O.unpermute_routing_map(r64, exp_idx, tokens.shape, p64, rmap, drop_and_pad=True)
+    exp.backward(g_out.double())
+    assert rel_l2(out, exp) <= TOL[dtype]
+    assert rel_l2(rows_d.grad, r64.grad) <= TOL[dtype]
+    assert rel_l2(probs_u.grad, p64.grad) <= TOL[dtype]
+
+
+def test_full_size_properties(device):
+    """Mixtral shape (4096 tokens, 8 experts, top-2, hidden 4096, bf16): size-independent properties."""
+    T, E, k, H = 4096, 8, 2, 4096
+    say("routing-map full size", T, E, k, H)
+    rmap, _ = make_map(T, E, k, 99)
+    gen = torch.Generator().manual_seed(5)
+    tokens = torch.randn(T, H, generator=gen).to(torch.bfloat16)
+    rmap_d, tok_d = rmap.to(device), tokens.to(device)
+    probs = torch.where(rmap_d, torch.full((T, E), 0.5, device=device), torch.zeros(T, E, device=device))
+    perm, pp, sidx = M.permute(tok_d, rmap_d, probs, fused=True)
+    counts = rmap.sum(0)
+    assert perm.size(0) == T * k and sidx.numel() == T * k
+    # expert-major, token-ascending inside every expert
+    s = sidx.cpu()
+    off = 0
+    for e in range(E):
+        seg = s[off:off + int(counts[e])]
+        assert torch.equal(seg, torch.nonzero(rmap[:, e]).view(-1))
+        off += int(counts[e])
+    assert torch.equal(perm, tok_d.index_select(0, sidx))
+    assert torch.all(pp == 0.5)
+    # round trip: weights 1/k give the tokens back exactly (two equal halves of a bf16 value)
+    back = M.unpermute(perm, sidx, tok_d.shape, probs=probs, routing_map=rmap_d, fused=True)
+    assert torch.equal(back, tok_d)
+
+
+def test_argument_checks(device):
+    tokens = torch.randn(4, 8, device=device)
+    rmap = torch.ones(4, 2, dtype=torch.bool, device=device)
+    with pytest.raises(TypeError):
+        M.permute(tokens, rmap.to(torch.int32))
+    with pytest.raises(RuntimeError):
+        M.permute(tokens, rmap[:3])
+    with pytest.raises(ValueError):
+        M.permute(tokens, rmap, drop_and_pad=True)
+    with pytest.raises(ValueError):
+        M.unpermute(torch.randn(8, 8, device=device), torch.zeros(8, dtype=torch.int64, device=device), tokens.shape)
+    with pytest.raises(RuntimeError):
+        M.permute(tokens.cpu(), rmap.cpu())

@@ -268,3 +268,75 @@ def test_plumbing_config_runs_and_is_consistent():
             sel = idx[:, j] == e
             dense[sel] += p[sel, j].double()[:, None] * y[sel]
     assert (out.double() - dense).norm() / dense.norm() < 1e-5
+
+
+# ---- routing-map (mask) mode ------------------------------------------------------------
+def _random_map(T, E, k, seed):
+    gen = torch.Generator().manual_seed(seed)
+    scores = torch.rand(T, E, generator=gen)
+    idx = scores.topk(k, dim=1).indices
+    rmap = torch.zeros(T, E, dtype=torch.bool)
+    rmap.scatter_(1, idx, True)
+    probs = torch.where(rmap, torch.rand(T, E, generator=gen) + 0.1, torch.zeros(T, E))
+    return rmap, probs, idx
+
+
+@pytest.mark.parametrize("T,E,k,seed", [(1, 1, 1, 0), (9, 4, 2, 1), (40, 8, 3, 2), (17, 5, 5, 3)])
+def test_routing_map_permute_bruteforce(T, E, k, seed):
+    rmap, probs, _ = _random_map(T, E, k, seed)
+    gen = torch.Generator().manual_seed(100 + seed)
+    tokens = torch.randn(T, 6, generator=gen)
+    permuted, pprobs, sidx = O.permute_routing_map(tokens, rmap, probs)
+    # brute force: expert-major, token-ascending
+    rows = [(e, t) for e in range(E) for t in range(T) if rmap[t, e]]
+    assert sidx.tolist() == [t for _, t in rows]
+    assert torch.equal(permuted, torch.stack([tokens[t] for _, t in rows]))
+    assert torch.equal(pprobs, torch.tensor([probs[t, e].item() for e, t in rows]))
+    # unpermute: out[t] = sum over its experts of probs * row
+    out = O.unpermute_routing_map(permuted, sidx, tokens.shape, probs, rmap)
+    want = torch.zeros(T, 6, dtype=torch.float64)
+    for r, (e, t) in enumerate(rows):
+        want[t] += probs[t, e].double() * permuted[r].double()
+    assert torch.allclose(out.double(), want, rtol=1e-6, atol=1e-6)
+    # without probs: plain sum of the rows of a token = k * token
+    out1 = O.unpermute_routing_map(permuted, sidx, tokens.shape)
+    assert torch.allclose(out1, tokens * k, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("T,E,k,cap,seed", [(9, 4, 2, 3, 1), (12, 3, 1, 6, 2), (10, 5, 2, 10, 3), (16, 4, 2, 1, 4)])
+def test_routing_map_drop_and_pad_bruteforce(T, E, k, cap, seed):
+    rmap, probs, _ = _random_map(T, E, k, seed)
+    gen = torch.Generator().manual_seed(200 + seed)
+    tokens = torch.randn(T, 5, generator=gen)
+    permuted, pprobs, sidx = O.permute_routing_map(tokens, rmap, probs, num_out_tokens=E * cap, drop_and_pad=True)
+    rows = []
+    for e in range(E):
+        routed = [t for t in range(T) if rmap[t, e]]
+        others = [t for t in range(T) if not rmap[t, e]]
+        rows += [(e, t) for t in (routed + others)[:cap]]
+    assert sidx.tolist() == [t for _, t in rows]
+    assert torch.equal(permuted, torch.stack([tokens[t] for _, t in rows]))
+    assert torch.equal(pprobs, torch.tensor([probs[t, e].item() for e, t in rows]))
+    out = O.unpermute_routing_map(permuted, sidx, tokens.shape, probs, rmap, drop_and_pad=True)
+    want = torch.zeros(T, 5, dtype=torch.float64)
+    for r, (e, t) in enumerate(rows):
+        want[t] += probs[t, e].double() * permuted[r].double()
+    assert torch.allclose(out.double(), want, rtol=1e-6, atol=1e-6)
+
+
+def test_routing_map_mode_agrees_with_index_mode():
+    # A map built from top-k indices: the mask form and the index form select the same multiset of rows per
+    # expert; with indices sorted inside every token they are the same permutation.
+    T, E, k = 50, 8, 2
+    rmap, probs, idx = _random_map(T, E, k, 7)
+    idx = idx.sort(dim=1).values
+    gen = torch.Generator().manual_seed(8)
+    tokens = torch.randn(T, 4, generator=gen)
+    p_idx, sorted_flat = O.permute(tokens, idx)
+    p_map, _, sidx = O.permute_routing_map(tokens, rmap)
+    assert torch.equal(p_idx, p_map)
+    assert torch.equal(sorted_flat // k, sidx)
+    topk_probs = probs.gather(1, idx)
+    out_idx = O.unpermute(p_idx, sorted_flat, topk_probs)
+    out_map = O.unpermute_routing_map(p_map, sidx, tokens.shape, probs, rmap)
+    assert torch.allclose(out_idx, out_map, rtol=1e-6, atol=1e-6)
