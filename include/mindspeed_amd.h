@@ -188,6 +188,20 @@ int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_strid
            int group_type, int64_t num_groups, int64_t m, int64_t k, int64_t n, int dtype,
            int out_dtype, int accumulate, void *workspace, size_t workspace_bytes);
 
+/* The same product (group_type 0 only) with one separately allocated weight matrix per group —
+ * the form torch_npu.npu_grouped_matmul([x], [w_0 .. w_{E-1}], ...) takes from
+ * mindspeed/te/pytorch/module/grouped_linear.py:61-69,85-93 (per-expert parameters
+ * weight0 .. weight{E-1}, :196-222).  weights: HOST array of num_groups device pointers; every
+ * matrix is [k, n] addressed with the same element strides (w_stride0, w_stride1), so the
+ * [n, k] parameters are read in place as transposed views.  At most 256 groups (the pointer
+ * differences travel as a kernel argument; stack the weights and use ms_gmm beyond that).
+ * Workspace size: ms_gmm_workspace_size. */
+int ms_gmm_weight_list(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1,
+                       const void *const *weights, int64_t w_stride0, int64_t w_stride1, void *y,
+                       int64_t y_stride_row, const int64_t *group_list, int group_list_type,
+                       int64_t num_groups, int64_t m, int64_t k, int64_t n, int dtype, int out_dtype,
+                       void *workspace, size_t workspace_bytes);
+
 /* ------------------------------------------------------------------------
  * SwiGLU (+ optional per-row probability) — stands in for the ATB
  * ACTIVATION_SWIGLU_FORWARD / BACKWARD calls of

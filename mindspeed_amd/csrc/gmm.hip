@@ -24,6 +24,17 @@
 namespace ms {
 namespace {
 
+// Per-group element offsets of separately allocated weight matrices, handed to the device as a kernel
+// argument (no host-to-device copy, so the call stays asynchronous and capturable).
+constexpr int kMaxWeightList = 256;
+struct WeightOffsets {
+    int64_t v[kMaxWeightList];
+};
+__global__ void gmm_weight_offsets_kernel(const WeightOffsets o, int n, int64_t *__restrict__ dst) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = o.v[i];
+}
+
 // ---- schedule ------------------------------------------------------------------------
 // With split_tails the last row tile of a group may be a smaller one (64 or 128 rows, the smallest that
 // holds the remainder), so ragged groups do not pay for a whole extra tile.  part = 0: one entry for the
@@ -62,7 +73,7 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
                                                            int m, int k, int tile_rows, int num_col_tiles,
                                                            int split_tails, int tails_last_below,
                                                            int64_t b_stride_group, int64_t c_stride_group,
-                                                           TileTable *table) {
+                                                           const int64_t *__restrict__ b_offsets, TileTable *table) {
     extern __shared__ int64_t gl[];
     for (int g = threadIdx.x; g < num_groups; g += blockDim.x) gl[g] = group_list[g];
     __syncthreads();
@@ -105,7 +116,7 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
                     e.row_end = static_cast<int>(end);
                     e.red_begin = 0;
                     e.red_end = k;
-                    e.b_off = g * b_stride_group;
+                    e.b_off = b_offsets != nullptr ? b_offsets[g] : g * b_stride_group;
                     e.c_off = 0;
                 } else {
                     e.row_begin = 0;
@@ -444,6 +455,9 @@ int current_device_cus() {
 size_t table_bytes(int64_t num_groups) {
     return sizeof(TileTable) + static_cast<size_t>(2 * num_groups + 2) * sizeof(GroupEntry);   // full + tail entries
 }
+// workspace = tile table, then (8-byte aligned) room for the per-group weight offsets of the list form
+size_t offsets_pos(int64_t num_groups) { return (table_bytes(num_groups) + 7) & ~static_cast<size_t>(7); }
+size_t workspace_need(int64_t num_groups) { return offsets_pos(num_groups) + kMaxWeightList * sizeof(int64_t); }
 
 template <int DT, int OUT>
 int launch16(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red, unsigned grid) {
@@ -472,15 +486,18 @@ extern "C" int ms_gmm_workspace_size(int64_t num_groups, int64_t m, int group_ty
     MS_REQUIRE(bytes != nullptr, MS_ERR_INVALID_ARGUMENT, "ms_gmm_workspace_size: bytes is NULL");
     MS_REQUIRE(num_groups >= 1 && num_groups <= kMaxGroups, MS_ERR_UNSUPPORTED,
                "ms_gmm_workspace_size: num_groups %lld outside [1, %d]", (long long)num_groups, kMaxGroups);
-    *bytes = (table_bytes(num_groups) + 255) & ~static_cast<size_t>(255);
+    *bytes = (workspace_need(num_groups) + 255) & ~static_cast<size_t>(255);
     return MS_OK;
 }
 
-extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int64_t x_stride1, const void *weight,
-                      int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1, void *y, int64_t y_stride_row,
-                      const int64_t *group_list, int group_list_type, int group_type, int64_t num_groups, int64_t m,
-                      int64_t k, int64_t n, int dtype, int out_dtype, int accumulate, void *workspace,
-                      size_t workspace_bytes) {
+// weight_offsets: nullptr for one strided weight tensor, else num_groups element offsets (relative to
+// `weight`) of separately allocated per-group matrices; all_weights_aligned16 then says whether every one of
+// them starts on a 16-byte boundary.
+static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64_t x_stride1, const void *weight,
+                    int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1, void *y, int64_t y_stride_row,
+                    const int64_t *group_list, int group_list_type, int group_type, int64_t num_groups, int64_t m,
+                    int64_t k, int64_t n, int dtype, int out_dtype, int accumulate, void *workspace,
+                    size_t workspace_bytes, const WeightOffsets *weight_offsets, bool all_weights_aligned16) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED, "ms_gmm: bad dtype %d", dtype);
     MS_REQUIRE(out_dtype == dtype || out_dtype == MS_FP32, MS_ERR_UNSUPPORTED,
@@ -494,7 +511,7 @@ extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int
     MS_REQUIRE(m >= 0 && k >= 0 && n >= 0 && m < (1ll << 31) - 512 && k < (1ll << 31) - 512 && n < (1ll << 31) - 512,
                MS_ERR_INVALID_ARGUMENT, "ms_gmm: bad sizes m=%lld k=%lld n=%lld", (long long)m, (long long)k, (long long)n);
     MS_REQUIRE(group_list != nullptr, MS_ERR_INVALID_ARGUMENT, "ms_gmm: group_list is NULL");
-    const size_t need = table_bytes(num_groups);
+    const size_t need = workspace_need(num_groups);
     MS_REQUIRE(workspace != nullptr && workspace_bytes >= need, MS_ERR_WORKSPACE_TOO_SMALL,
                "ms_gmm: workspace %zu < %zu bytes", workspace_bytes, need);
     MS_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7u) == 0, MS_ERR_INVALID_ARGUMENT, "ms_gmm: workspace must be 8-byte aligned");
@@ -529,11 +546,18 @@ extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int
     TileTable *table = static_cast<TileTable *>(workspace);
     const int64_t c_stride_group = k * y_stride_row;
     const int num_cus = current_device_cus();
+    int64_t *b_offsets = nullptr;
+    if (weight_offsets != nullptr) {
+        b_offsets = reinterpret_cast<int64_t *>(static_cast<char *>(workspace) + offsets_pos(num_groups));
+        hipLaunchKernelGGL(gmm_weight_offsets_kernel, dim3(1), dim3(kMaxWeightList), 0, stream, *weight_offsets,
+                           static_cast<int>(num_groups), b_offsets);
+        MS_CHECK_LAUNCH("gmm_weight_offsets_kernel");
+    }
     auto schedule = [&](int split_tails) -> int {
         hipLaunchKernelGGL(gmm_schedule_kernel, dim3(1), dim3(256), static_cast<size_t>(num_groups) * sizeof(int64_t),
                            stream, group_list, group_list_type, group_type, static_cast<int>(num_groups),
                            static_cast<int>(m), static_cast<int>(k), tile_rows, static_cast<int>(num_col_tiles),
-                           split_tails, kTailsLastRounds * num_cus, w_stride_group, c_stride_group, table);
+                           split_tails, kTailsLastRounds * num_cus, w_stride_group, c_stride_group, b_offsets, table);
         MS_CHECK_LAUNCH("gmm_schedule_kernel");
         return MS_OK;
     };
@@ -568,7 +592,8 @@ extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int
     const int64_t a_other = use_a_red ? a_stride_row : a_stride_red;
     const int64_t b_other = use_b_red ? b_stride_col : b_stride_red;
     args.a_vec_ok = aligned16(x) && a_other % 8 == 0;
-    args.b_vec_ok = aligned16(weight) && b_other % 8 == 0 && w_stride_group % 8 == 0;
+    args.b_vec_ok = weight_offsets != nullptr ? (all_weights_aligned16 && b_other % 8 == 0)
+                                              : (aligned16(weight) && b_other % 8 == 0 && w_stride_group % 8 == 0);
     const int out_size = out_dtype == MS_FP32 ? 4 : 2;
     args.c_vec_ok = (reinterpret_cast<uintptr_t>(y) % (4 * out_size) == 0) && y_stride_row % 4 == 0 &&
                     (group_type == 0 || c_stride_group % 4 == 0);
@@ -602,4 +627,42 @@ extern "C" int ms_gmm(ms_stream_t stream_, const void *x, int64_t x_stride0, int
     if (out == OUT_SAME) return launch16<MS_FP16, OUT_SAME>(stream, args, a_is_red, b_is_red, grid);
     if (out == OUT_F32) return launch16<MS_FP16, OUT_F32>(stream, args, a_is_red, b_is_red, grid);
     return launch16<MS_FP16, ACC_F32>(stream, args, a_is_red, b_is_red, grid);
+}
+
+extern "C" int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1, const void *weight,
+                      int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1, void *y, int64_t y_stride_row,
+                      const int64_t *group_list, int group_list_type, int group_type, int64_t num_groups, int64_t m,
+                      int64_t k, int64_t n, int dtype, int out_dtype, int accumulate, void *workspace,
+                      size_t workspace_bytes) {
+    return gmm_impl(stream, x, x_stride0, x_stride1, weight, w_stride_group, w_stride0, w_stride1, y, y_stride_row,
+                    group_list, group_list_type, group_type, num_groups, m, k, n, dtype, out_dtype, accumulate,
+                    workspace, workspace_bytes, nullptr, false);
+}
+
+extern "C" int ms_gmm_weight_list(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1,
+                                  const void *const *weights, int64_t w_stride0, int64_t w_stride1, void *y,
+                                  int64_t y_stride_row, const int64_t *group_list, int group_list_type,
+                                  int64_t num_groups, int64_t m, int64_t k, int64_t n, int dtype, int out_dtype,
+                                  void *workspace, size_t workspace_bytes) {
+    MS_REQUIRE(num_groups >= 1 && num_groups <= kMaxWeightList, MS_ERR_UNSUPPORTED,
+               "ms_gmm_weight_list: num_groups %lld outside [1, %d] (stack the weights and use ms_gmm beyond that)",
+               (long long)num_groups, kMaxWeightList);
+    MS_REQUIRE(weights != nullptr, MS_ERR_INVALID_ARGUMENT, "ms_gmm_weight_list: weights is NULL");
+    MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED,
+               "ms_gmm_weight_list: bad dtype %d", dtype);
+    const int64_t elem = dtype == MS_FP32 ? 4 : 2;
+    WeightOffsets off{};
+    bool aligned = true;
+    for (int64_t g = 0; g < num_groups; ++g) {
+        MS_REQUIRE(weights[g] != nullptr || k == 0 || n == 0, MS_ERR_INVALID_ARGUMENT,
+                   "ms_gmm_weight_list: weights[%lld] is NULL", (long long)g);
+        const int64_t delta = static_cast<const char *>(weights[g]) - static_cast<const char *>(weights[0]);
+        MS_REQUIRE(delta % elem == 0, MS_ERR_INVALID_ARGUMENT,
+                   "ms_gmm_weight_list: weights[%lld] is not element-aligned relative to weights[0]", (long long)g);
+        off.v[g] = delta / elem;
+        aligned = aligned && aligned16(weights[g]);
+    }
+    return gmm_impl(stream, x, x_stride0, x_stride1, weights[0], 0, w_stride0, w_stride1, y, y_stride_row, group_list,
+                    group_list_type, /*group_type=*/0, num_groups, m, k, n, dtype, out_dtype, /*accumulate=*/0,
+                    workspace, workspace_bytes, &off, aligned);
 }
