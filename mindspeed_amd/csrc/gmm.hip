@@ -5,20 +5,18 @@
 // Structure
 //   * gmm_schedule_kernel turns the device-resident group_list into a table of
 //     per-group tile ranges (no host read of group_list, empty groups emit no
-//     row tiles, a trailing pseudo-group zero-fills rows past the last offset).
-//   * gmm16_kernel: bf16 / fp16, 256x256x64 macro tile per 256-thread workgroup
-//     (2x2 wavefronts, 128x128 per wavefront = 4x4 v_mfma_f32_32x32x16), fp32
-//     accumulators, LDS double buffer (128 KB of the CU's 160 KB), operands
-//     stored in LDS as [outer][reduction] with an XOR swizzle of the 16-byte
-//     chunks so ds_read_b128 fragment loads are bank-conflict free.  Operands
-//     whose contiguous memory dim is not the reduction dim are transposed in
-//     registers (8x8 blocks) on their way from global memory to LDS, so NN, NT
-//     and TN products all run the same inner loop.
-//   * tiles are rasterised per XCD: workgroup b runs on XCD b%8, each XCD owns a
-//     contiguous range of logical tiles ordered row-tile-fastest inside a column
-//     panel, so concurrently running workgroups of an XCD share weight panels
-//     in that XCD's L2.
-//   * gmm32_kernel: fp32 inputs, v_mfma_f32_32x32x2f32, 128x128x8 tiles.
+//     row tiles, a trailing pseudo-group zero-fills rows past the last offset;
+//     ragged groups may end in a 64- or 128-row tile; per-group weight offsets
+//     may come from a list of separately allocated matrices).
+//   * every XCD takes a contiguous eighth of every group's tiles (workgroup b
+//     runs on XCD b % 8), row-tile-fastest inside a column panel, so the
+//     workgroups running together on an XCD share operand panels in its L2.
+//   * the fast 16-bit kernels live in gmm_fast.hip.  Here: gmm16_kernel, the
+//     16-bit kernel for operands that do not allow 16-byte vector access
+//     (element-wise guarded loads, operands that are not contiguous along the
+//     reduction dim transposed in registers on their way to LDS), same
+//     256x256x64 tile and 4x4 v_mfma_f32_32x32x16 per wavefront; and
+//     gmm32_kernel for fp32 inputs (v_mfma_f32_32x32x2f32, 128x128x8 tiles).
 #include "gmm_common.h"
 
 namespace ms {
