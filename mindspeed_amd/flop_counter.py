@@ -80,6 +80,12 @@ def record(timing=True):
         _active = prev
 
 
+def timing_active() -> bool:
+    """True while a recorder is bracketing every op with events (ops then keep to one stream, so that the
+    per-op durations are those of kernels running alone)."""
+    return _active is not None and _active.timing
+
+
 @contextlib.contextmanager
 def op(name, work, unit, device):
     """Used by the ops around each C-ABI call; free when no Recorder is active."""

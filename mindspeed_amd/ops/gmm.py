@@ -12,6 +12,7 @@ transposed in memory.
 from __future__ import annotations
 
 import ctypes
+import os
 
 import torch
 
@@ -157,6 +158,55 @@ def gmm_raw_weight_list(x, weights, group_list, group_list_type, transposed=Fals
     return out
 
 
+# dX and dW of one grouped matmul are independent; each is a full-chip kernel whose last round of tiles leaves
+# compute units idle.  With OVERLAP_WGRAD the weight-gradient product is launched on a second stream (default
+# priority) between two joins with the caller's stream, so its tiles fill the other kernel's tail and vice versa.
+OVERLAP_WGRAD = os.environ.get("MINDSPEED_AMD_OVERLAP_WGRAD", "1") != "0"
+_side_streams = {}
+
+
+def _side_stream(device) -> torch.cuda.Stream:
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    s = _side_streams.get(key)
+    if s is None:
+        s = torch.cuda.Stream(device=device)
+        _side_streams[key] = s
+    return s
+
+
+class _beside:
+    """``with _beside(device) as side:`` runs the body on the side stream after everything queued so far on the
+    current stream; ``side.join(*tensors)`` (call it after queueing the main-stream work that should overlap)
+    makes the current stream wait for the body and hands the tensors over to it.  Without overlap (disabled,
+    or while ops are being event-timed one by one) the body simply runs on the current stream."""
+
+    def __init__(self, device):
+        self.device = device
+        self.active = OVERLAP_WGRAD and not flop_counter.timing_active()
+        self.main = torch.cuda.current_stream(device)
+        self.side = _side_stream(device) if self.active else None
+        self.ctx = None
+
+    def __enter__(self):
+        if self.active:
+            self.side.wait_stream(self.main)
+            self.ctx = torch.cuda.stream(self.side)
+            self.ctx.__enter__()
+        return self
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
+
+    def join(self, *tensors):
+        if self.active:
+            self.main.wait_stream(self.side)
+            for t in tensors:
+                if t is not None:
+                    t.record_stream(self.main)
+
+
 class _RawGmmModule:
     """Stand-in for the pybind module of mindspeed/ops/csrc/cann/gmm.cpp:295-309.
 
@@ -178,8 +228,10 @@ class _RawGmmModule:
     def npu_gmm_backward(grad, x, weight, group_list, group_list_type):
         # gmm.cpp:169-246: dx = gmm(grad, w^T, 0); dw = gmm(x^T, grad, 2).reshape(w.shape)
         glt = group_list_type or 0
+        with _beside(grad[0].device) as side:
+            dw = gmm_raw(x[0].transpose(-1, -2), grad[0], group_list, 2, glt).reshape(weight[0].shape)
         dx = gmm_raw(grad[0], weight[0].transpose(-1, -2), group_list, 0, glt)
-        dw = gmm_raw(x[0].transpose(-1, -2), grad[0], group_list, 2, glt).reshape(weight[0].shape)
+        side.join(dw)
         return [dx], [dw], []
 
     @staticmethod
@@ -240,12 +292,14 @@ class GMMFunction(torch.autograd.Function):
         module = GMMFunction.builder.load() if ctx.group_list_type == 0 else GMMFunction.builder2.load()
 
         if ctx.gemm_fusion:
+            with _beside(grad_outputs.device) as side:
+                if ctx.group_list_type == 0:
+                    cumulative = group_list
+                else:
+                    cumulative = torch.cumsum(group_list, dim=0)
+                npu_groupmatmul_add_fp32(x, grad_outputs, cumulative, original_weight.main_grad)
             dx, _, dbias = module.npu_gmm_backward_fusion([grad_outputs], [weight], group_list, ctx.group_list_type)
-            if ctx.group_list_type == 0:
-                cumulative = group_list
-            else:
-                cumulative = torch.cumsum(group_list, dim=0)
-            npu_groupmatmul_add_fp32(x, grad_outputs, cumulative, original_weight.main_grad)
+            side.join()
             dbias = None if len(dbias) == 0 else dbias[0]
             if hasattr(original_weight, "grad_added_to_main_grad"):
                 if getattr(weight, "zero_out_wgrad", False):
