@@ -45,7 +45,8 @@ def gmm_raw(x, weight, group_list, group_type, group_list_type, out=None, accumu
 
     group_type 0: ``x [M, K]``, ``weight [E, K, N]`` -> ``[M, N]``.
     group_type 2: ``x [K, M]``, ``weight [M, N]`` -> ``[E, K, N]``.
-    ``out`` (fp32, contiguous) with ``accumulate`` adds the result in place.
+    ``out``: optional preallocated contiguous result (fp32, or x's dtype); fp32 with ``accumulate`` adds the
+    result in place.
     """
     lib = _lib.load()
     _lib.require_device(x, "x")
@@ -84,9 +85,12 @@ def gmm_raw(x, weight, group_list, group_type, group_list_type, out=None, accumu
         out = torch.empty(out_shape, dtype=x.dtype, device=dev)
         out_dtype = dtype
     else:
-        if out.dtype != torch.float32 or not out.is_contiguous() or out.numel() != out_shape[0] * out_shape[1] * (out_shape[2] if len(out_shape) == 3 else 1):
-            raise ValueError("out must be a contiguous fp32 tensor of the result's size")
-        out_dtype = _lib.MS_FP32
+        numel = out_shape[0] * out_shape[1] * (out_shape[2] if len(out_shape) == 3 else 1)
+        if out.dtype not in (torch.float32, x.dtype) or not out.is_contiguous() or out.numel() != numel:
+            raise ValueError("out must be a contiguous tensor of the result's size, fp32 or of x's dtype")
+        if accumulate and out.dtype != torch.float32:
+            raise ValueError("accumulate needs an fp32 out")
+        out_dtype = _lib.MS_FP32 if out.dtype == torch.float32 else dtype
     nbytes = ctypes.c_size_t(0)
     _lib.check(lib.ms_gmm_workspace_size(num_groups, m, group_type, ctypes.byref(nbytes)), "ms_gmm_workspace_size")
     ws = _lib.workspace(nbytes.value, dev)
@@ -176,8 +180,9 @@ def _side_stream(device) -> torch.cuda.Stream:
 
 class _beside:
     """``with _beside(device) as side:`` runs the body on the side stream after everything queued so far on the
-    current stream; ``side.join(*tensors)`` (call it after queueing the main-stream work that should overlap)
-    makes the current stream wait for the body and hands the tensors over to it.  Without overlap (disabled,
+    current stream; ``side.join()`` (call it after queueing the main-stream work that should overlap)
+    makes the current stream wait for the body.  Results of the body should live in memory that was
+    allocated on the caller's stream beforehand.  Without overlap (disabled,
     or while ops are being event-timed one by one) the body simply runs on the current stream."""
 
     def __init__(self, device):
@@ -199,12 +204,9 @@ class _beside:
             self.ctx.__exit__(*exc)
         return False
 
-    def join(self, *tensors):
+    def join(self):
         if self.active:
             self.main.wait_stream(self.side)
-            for t in tensors:
-                if t is not None:
-                    t.record_stream(self.main)
 
 
 class _RawGmmModule:
@@ -228,11 +230,17 @@ class _RawGmmModule:
     def npu_gmm_backward(grad, x, weight, group_list, group_list_type):
         # gmm.cpp:169-246: dx = gmm(grad, w^T, 0); dw = gmm(x^T, grad, 2).reshape(w.shape)
         glt = group_list_type or 0
+        # The result is allocated on the caller's stream: a block that belonged to the side stream's pool
+        # would have its release deferred until the caller's stream is done with it, and the next step's
+        # request on the side stream would then go to the driver for fresh memory.
+        w = weight[0]
+        num_groups = len(group_list) if not isinstance(group_list, torch.Tensor) else group_list.numel()
+        dw = torch.empty((num_groups, x[0].size(-1), grad[0].size(-1)), dtype=x[0].dtype, device=x[0].device)
         with _beside(grad[0].device) as side:
-            dw = gmm_raw(x[0].transpose(-1, -2), grad[0], group_list, 2, glt).reshape(weight[0].shape)
-        dx = gmm_raw(grad[0], weight[0].transpose(-1, -2), group_list, 0, glt)
-        side.join(dw)
-        return [dx], [dw], []
+            gmm_raw(x[0].transpose(-1, -2), grad[0], group_list, 2, glt, out=dw)
+        dx = gmm_raw(grad[0], w.transpose(-1, -2), group_list, 0, glt)
+        side.join()
+        return [dx], [dw.reshape(w.shape)], []
 
     @staticmethod
     def npu_gmm_backward_fusion(grad, weight, group_list, group_list_type):
