@@ -534,6 +534,99 @@ __global__ void copy_tail_kernel(const unsigned char *src, unsigned char *dst, s
     if (i < end) dst[i] = src[i];
 }
 
+// ---- sort + row scatter in one launch (small inputs, few bins) ------------------------------------
+// The single-workgroup sort is latency, not work: ~12 us for 8192 keys, after which the row scatter still has to
+// be launched.  Here every scatter workgroup works out the rows of its own tokens itself: its four wavefronts
+// count, per bin, the keys in front of the workgroup's first flat position and the keys from there on (two
+// histograms over all keys, read from L2 after the first workgroup has touched them), a scan over the bins
+// turns that into each bin's next free row as seen from this workgroup, and wavefront 0 ranks the
+// workgroup's own positions with the same stable scatter the sort kernels use.  Counting is redundant across
+// workgroups (every one reads all keys) but cheap, and it overlaps with the row traffic of the workgroups
+// that are already copying.  The integer outputs are the same as the sort kernels' by construction.
+constexpr int kFusedMaxBins = 16;   // the per-bin ballot counting; measured slower than two launches with 1024 bins
+
+template <typename IdxT, typename VecT>
+__global__ __launch_bounds__(256) void permute_fused_kernel(
+    const VecT *__restrict__ tokens, VecT *__restrict__ permuted, const IdxT *__restrict__ idx, int n, int nbins,
+    int nbits, int num_out, int32_t *__restrict__ row_id_map, int32_t *__restrict__ sorted_indices,
+    int64_t *__restrict__ tokens_per_expert, int tpe_n, int num_tokens, int topk, int vecs_per_row, int lanes) {
+    extern __shared__ int lds[];               // before[4][nbins], after[4][nbins], base[nbins], 16 ints scratch
+    int *before = lds;
+    int *after = lds + 4 * nbins;
+    int *base = lds + 8 * nbins;
+    int *scratch = base + nbins;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int rows_per_block = 256 / lanes;
+    const int t0 = blockIdx.x * rows_per_block;
+    const int t1 = min(t0 + rows_per_block, num_tokens);
+    const int p0 = t0 * topk, p1 = t1 * topk;  // this workgroup's flat positions
+    for (int i = tid; i < 8 * nbins; i += 256) lds[i] = 0;
+    __syncthreads();
+    int seg = (n + 3) / 4;
+    seg = (seg + 63) & ~63;
+    const int b = min(wave * seg, n);
+    const int e = min(b + seg, n);
+    const int mid = min(max(p0, b), e);
+    wave_histogram(before + wave * nbins, idx, b, mid, nbins, nbits);
+    wave_histogram(after + wave * nbins, idx, mid, e, nbins, nbits);
+    __syncthreads();
+    // bins in passes of 256 (one per thread), the running row count carried from pass to pass
+    int carry = 0;
+    for (int e0 = 0; e0 < nbins; e0 += 256) {
+        const int bin = e0 + tid;
+        int bef = 0, tot = 0;
+        if (bin < nbins) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                bef += before[w * nbins + bin];
+                tot += after[w * nbins + bin];
+            }
+            tot += bef;
+        }
+        const int first = carry + block_exclusive_scan(tot, scratch);   // first row of this bin
+        if (bin < nbins) {
+            base[bin] = first + bef;
+            if (blockIdx.x == 0 && tokens_per_expert != nullptr && bin < tpe_n) tokens_per_expert[bin] = tot;
+        }
+        if (tid == 255) scratch[15] = first + tot;
+        __syncthreads();
+        carry = scratch[15];
+        __syncthreads();
+    }
+    if (wave == 0) wave_scatter(base, idx, p0, p1, nbins, nbits, num_out, row_id_map, sorted_indices);
+    // Workgroup-scope release / acquire (part of __syncthreads) is all the other wavefronts need to see the
+    // row ids: they run on the same compute unit.  A device-scope fence here would write the L2 back, rows
+    // of other workgroups included, once per workgroup.
+    __syncthreads();
+
+    const int local_row = tid / lanes;
+    const int lane = tid % lanes;
+    const int t = t0 + local_row;
+    if (t >= num_tokens) return;
+    const VecT *src = tokens + static_cast<int64_t>(t) * vecs_per_row;
+    for (int j0 = 0; j0 < topk; j0 += kSlotBatch) {
+        int d[kSlotBatch];
+#pragma unroll
+        for (int j = 0; j < kSlotBatch; ++j)
+            d[j] = j0 + j < topk ? row_id_map[static_cast<int64_t>(t) * topk + j0 + j] : num_out;
+        for (int c0 = lane; c0 < vecs_per_row; c0 += 4 * lanes) {
+            VecT v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
+#pragma unroll
+            for (int j = 0; j < kSlotBatch; ++j) {
+                if (static_cast<unsigned>(d[j]) >= static_cast<unsigned>(num_out)) continue;   // dropped (or corrupt) id
+                VecT *dst = permuted + static_cast<int64_t>(d[j]) * vecs_per_row;
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (c0 + u * lanes < vecs_per_row) dst[c0 + u * lanes] = v[u];
+            }
+        }
+    }
+}
+
 // ---- routing-map (mask) mode ----------------------------------------------------------
 // The [T, E] boolean routing map is sorted with the same counting sort as the index form: flat position
 // i = t*E + e gets the key e when the entry is set and the extra last key E when it is not, so the set
@@ -672,6 +765,36 @@ int launch_permute_rows(hipStream_t stream, const void *tokens, void *permuted, 
     return MS_OK;
 }
 
+template <typename IdxT, typename VecT>
+int launch_permute_fused(hipStream_t stream, const SortPlan &p, const void *tokens, void *permuted, const IdxT *idx,
+                         int num_out, int32_t *row_id_map, int32_t *sorted_indices, int64_t *tpe, int tpe_n,
+                         int64_t T, int64_t k, int64_t row_bytes) {
+    const int64_t vecs = row_bytes / sizeof(VecT);
+    const RowLayout rl = row_layout(vecs);
+    const int64_t blocks = ceil_div(T, rl.rows_per_block);
+    const size_t lds = (static_cast<size_t>(9) * p.nbins + 16) * sizeof(int);
+    hipLaunchKernelGGL((permute_fused_kernel<IdxT, VecT>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, stream,
+                       static_cast<const VecT *>(tokens), static_cast<VecT *>(permuted), idx, p.n, p.nbins, p.nbits,
+                       num_out, row_id_map, sorted_indices, tpe, tpe_n, static_cast<int>(T), static_cast<int>(k),
+                       static_cast<int>(vecs), rl.lanes);
+    MS_CHECK_LAUNCH("permute_fused_kernel");
+    return MS_OK;
+}
+
+template <typename IdxT>
+int permute_fused_dispatch(hipStream_t stream, const SortPlan &p, const void *tokens, void *permuted, const IdxT *idx,
+                           int num_out, int32_t *row_id_map, int32_t *sorted_indices, int64_t *tpe, int tpe_n,
+                           int64_t T, int64_t k, int64_t row_bytes, int dtype) {
+    if (row_bytes % 16 == 0 && aligned16(tokens) && aligned16(permuted))
+        return launch_permute_fused<IdxT, v16>(stream, p, tokens, permuted, idx, num_out, row_id_map, sorted_indices, tpe,
+                                               tpe_n, T, k, row_bytes);
+    if (dtype == MS_FP32)
+        return launch_permute_fused<IdxT, uint32_t>(stream, p, tokens, permuted, idx, num_out, row_id_map, sorted_indices,
+                                                    tpe, tpe_n, T, k, row_bytes);
+    return launch_permute_fused<IdxT, uint16_t>(stream, p, tokens, permuted, idx, num_out, row_id_map, sorted_indices, tpe,
+                                                tpe_n, T, k, row_bytes);
+}
+
 template <typename DT>
 int launch_gather_combine(hipStream_t stream, const void *rows, const int32_t *map, const void *probs, void *out,
                           int64_t T, int64_t k, int64_t H, int64_t num_rows) {
@@ -772,6 +895,16 @@ extern "C" int ms_moe_token_permute(ms_stream_t stream_, const void *tokens, con
     const size_t need = p.small ? 0 : static_cast<size_t>(p.nseg) * p.nbins * sizeof(int);
     MS_REQUIRE(workspace_bytes >= need && (need == 0 || workspace != nullptr), MS_ERR_WORKSPACE_TOO_SMALL,
                "ms_moe_token_permute: workspace %zu < %zu bytes", workspace_bytes, need);
+    const int64_t row_bytes = H * dtype_size(dtype);
+    // small inputs with a known, modest number of experts: sort and row scatter in one launch
+    if (p.small && p.nbins <= kFusedMaxBins && num_out > 0) {
+        if (index_dtype == MS_INT32)
+            return permute_fused_dispatch(stream, p, tokens, permuted, static_cast<const int32_t *>(indices), (int)num_out,
+                                          row_id_map, sorted_indices, tokens_per_expert, (int)experts_hint, T, k, row_bytes,
+                                          dtype);
+        return permute_fused_dispatch(stream, p, tokens, permuted, static_cast<const int64_t *>(indices), (int)num_out,
+                                      row_id_map, sorted_indices, tokens_per_expert, (int)experts_hint, T, k, row_bytes, dtype);
+    }
     int rc;
     if (index_dtype == MS_INT32)
         rc = launch_sort(stream, p, static_cast<const int32_t *>(indices), (int)num_out, row_id_map, sorted_indices,
@@ -781,7 +914,6 @@ extern "C" int ms_moe_token_permute(ms_stream_t stream_, const void *tokens, con
                          tokens_per_expert, (int)experts_hint, workspace);
     if (rc) return rc;
     if (num_out == 0) return MS_OK;
-    const int64_t row_bytes = H * dtype_size(dtype);
     if (row_bytes % 16 == 0 && aligned16(tokens) && aligned16(permuted))
         return launch_permute_rows<v16>(stream, tokens, permuted, row_id_map, T, k, row_bytes, num_out);
     if (dtype == MS_FP32) return launch_permute_rows<uint32_t>(stream, tokens, permuted, row_id_map, T, k, row_bytes, num_out);
