@@ -188,6 +188,21 @@ int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_strid
            int group_type, int64_t num_groups, int64_t m, int64_t k, int64_t n, int dtype,
            int out_dtype, int accumulate, void *workspace, size_t workspace_bytes);
 
+/* First grouped matmul of an expert MLP with the SwiGLU (x per-row probability) activation fused into
+ * its epilogue: the op sequence fc1 = gmm(x, w1); act = (silu(gate) * up * probs).to(dtype) of
+ * mindspeed/core/transformer/moe/moe_feature/gmm/experts.py:113-127 (activation: :41-44) in one launch.
+ * weight [num_groups, k, 2*ffn] (gate columns first); y [m, 2*ffn] receives the fc1 output (kept
+ * for backward; may be NULL), act [m, ffn] the activation, computed from the rounded fc1 values
+ * exactly as ms_swiglu computes it from y.  probs: optional [m] (bf16 / fp16 / fp32).  group_type 0
+ * only; bf16 / fp16; needs the vector-access layout (16-byte aligned pointers, x contiguous along k,
+ * weight contiguous along its columns, k, ffn and all strides multiples of 8) and reports
+ * MS_ERR_UNSUPPORTED otherwise.  Workspace size: ms_gmm_workspace_size. */
+int ms_gmm_swiglu(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1,
+                  const void *weight, int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1,
+                  void *y, int64_t y_stride_row, void *act, int64_t act_stride_row, const void *probs,
+                  int probs_dtype, const int64_t *group_list, int group_list_type, int64_t num_groups,
+                  int64_t m, int64_t k, int64_t ffn, int dtype, void *workspace, size_t workspace_bytes);
+
 /* The same product (group_type 0 only) with one separately allocated weight matrix per group —
  * the form torch_npu.npu_grouped_matmul([x], [w_0 .. w_{E-1}], ...) takes from
  * mindspeed/te/pytorch/module/grouped_linear.py:61-69,85-93 (per-expert parameters

@@ -491,11 +491,20 @@ extern "C" int ms_gmm_workspace_size(int64_t num_groups, int64_t m, int group_ty
 // weight_offsets: nullptr for one strided weight tensor, else num_groups element offsets (relative to
 // `weight`) of separately allocated per-group matrices; all_weights_aligned16 then says whether every one of
 // them starts on a 16-byte boundary.
+// Second output of the fused SwiGLU form (n = 2 * ffn weight columns: gate | up).
+struct SwigluOut {
+    void *act;
+    int64_t act_stride_row;
+    const void *probs;
+    int probs_dtype;
+};
+
 static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64_t x_stride1, const void *weight,
                     int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1, void *y, int64_t y_stride_row,
                     const int64_t *group_list, int group_list_type, int group_type, int64_t num_groups, int64_t m,
                     int64_t k, int64_t n, int dtype, int out_dtype, int accumulate, void *workspace,
-                    size_t workspace_bytes, const WeightOffsets *weight_offsets, bool all_weights_aligned16) {
+                    size_t workspace_bytes, const WeightOffsets *weight_offsets, bool all_weights_aligned16,
+                    const SwigluOut *swiglu = nullptr) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED, "ms_gmm: bad dtype %d", dtype);
     MS_REQUIRE(out_dtype == dtype || out_dtype == MS_FP32, MS_ERR_UNSUPPORTED,
@@ -518,7 +527,7 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     const int64_t out_rows = group_type == 0 ? m : k;       // rows per output block
     const int64_t red_total = group_type == 0 ? k : m;
     if (n == 0 || out_rows == 0) return MS_OK;
-    MS_REQUIRE(y != nullptr, MS_ERR_INVALID_ARGUMENT, "ms_gmm: y is NULL");
+    MS_REQUIRE(y != nullptr || swiglu != nullptr, MS_ERR_INVALID_ARGUMENT, "ms_gmm: y is NULL");
     MS_REQUIRE(red_total == 0 || (x != nullptr && weight != nullptr), MS_ERR_INVALID_ARGUMENT, "ms_gmm: NULL operand");
     MS_REQUIRE(y_stride_row >= n, MS_ERR_INVALID_ARGUMENT, "ms_gmm: y_stride_row %lld < n %lld", (long long)y_stride_row, (long long)n);
 
@@ -535,7 +544,8 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     const bool is32 = dtype == MS_FP32;
     const int tile_rows = is32 ? FM : BM;
     const int tile_cols = is32 ? FN : BN;
-    const int64_t num_col_tiles = ceil_div(n, tile_cols);
+    // fused SwiGLU form: a tile holds 128 gate and the matching 128 up columns, i.e. 128 activation columns
+    const int64_t num_col_tiles = swiglu != nullptr ? ceil_div(n / 2, tile_cols / 2) : ceil_div(n, tile_cols);
     const int64_t row_tiles_bound = group_type == 0 ? ceil_div(m, tile_rows) + num_groups + 2
                                                     : num_groups * (k / tile_rows + 1);
     const int64_t tiles_bound = row_tiles_bound * num_col_tiles;
@@ -574,7 +584,15 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     args.num_col_tiles = static_cast<int>(num_col_tiles);
     const unsigned grid = static_cast<unsigned>((ceil_div(tiles_bound, 8) + 2 * num_groups + 2) * 8);
 
+    if (swiglu != nullptr) {
+        args.cols = static_cast<int>(n / 2);
+        args.act = swiglu->act;
+        args.act_stride_row = swiglu->act_stride_row;
+        args.probs = swiglu->probs;
+        args.probs_dtype = swiglu->probs_dtype;
+    }
     if (is32) {
+        MS_REQUIRE(swiglu == nullptr, MS_ERR_UNSUPPORTED, "ms_gmm_swiglu: 16-bit dtypes only");
         if (int rc = schedule(0)) return rc;
         if (accumulate)
             hipLaunchKernelGGL(gmm32_kernel<true>, dim3(grid), dim3(256), 0, stream, args);
@@ -595,6 +613,9 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     const int out_size = out_dtype == MS_FP32 ? 4 : 2;
     args.c_vec_ok = (reinterpret_cast<uintptr_t>(y) % (4 * out_size) == 0) && y_stride_row % 4 == 0 &&
                     (group_type == 0 || c_stride_group % 4 == 0);
+    if (swiglu != nullptr)   // 16-byte row stores of both outputs, whole 8-column chunks in each half
+        args.c_vec_ok = aligned16(y) && y_stride_row % 8 == 0 && aligned16(swiglu->act) &&
+                        swiglu->act_stride_row % 8 == 0 && (n / 2) % 8 == 0;
     // A stride of 1 in a dim of extent 1 may come with an arbitrary other stride.
     const bool a_is_red = use_a_red || !a_row;
     const bool b_is_red = use_b_red || !b_col;
@@ -615,6 +636,13 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     const int64_t a_span = a_is_red ? 256 * a_stride_row : 64 * a_stride_red;
     const int64_t b_span = b_is_red ? 256 * b_stride_col : 64 * b_stride_red;
     fast = fast && a_span < (1ll << 30) && b_span < (1ll << 30);
+    if (swiglu != nullptr) {
+        MS_REQUIRE(fast && a_is_red && !b_is_red, MS_ERR_UNSUPPORTED,
+                   "ms_gmm_swiglu: needs the vector-access layout (16-byte aligned operands and outputs, x contiguous "
+                   "along k, weight contiguous along its columns, k and ffn multiples of 8)");
+        if (int rc = schedule(1)) return rc;
+        return launch_gmm16_fast(stream, args, dtype, OUT_SWIGLU, true, false, grid);
+    }
     if (int rc = schedule(fast ? 1 : 0)) return rc;
     if (fast) return launch_gmm16_fast(stream, args, dtype, out, a_is_red, b_is_red, grid);
     if (dtype == MS_BF16) {
@@ -635,6 +663,24 @@ extern "C" int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int6
     return gmm_impl(stream, x, x_stride0, x_stride1, weight, w_stride_group, w_stride0, w_stride1, y, y_stride_row,
                     group_list, group_list_type, group_type, num_groups, m, k, n, dtype, out_dtype, accumulate,
                     workspace, workspace_bytes, nullptr, false);
+}
+
+extern "C" int ms_gmm_swiglu(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1, const void *weight,
+                             int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1, void *y, int64_t y_stride_row,
+                             void *act, int64_t act_stride_row, const void *probs, int probs_dtype,
+                             const int64_t *group_list, int group_list_type, int64_t num_groups, int64_t m, int64_t k,
+                             int64_t ffn, int dtype, void *workspace, size_t workspace_bytes) {
+    MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16, MS_ERR_UNSUPPORTED, "ms_gmm_swiglu: dtype must be bf16 or fp16");
+    MS_REQUIRE(ffn >= 0 && ffn < (1ll << 30), MS_ERR_INVALID_ARGUMENT, "ms_gmm_swiglu: bad ffn %lld", (long long)ffn);
+    MS_REQUIRE(act != nullptr || m == 0 || ffn == 0, MS_ERR_INVALID_ARGUMENT, "ms_gmm_swiglu: act is NULL");
+    MS_REQUIRE(act_stride_row >= ffn, MS_ERR_INVALID_ARGUMENT, "ms_gmm_swiglu: act_stride_row %lld < ffn %lld",
+               (long long)act_stride_row, (long long)ffn);
+    MS_REQUIRE(probs == nullptr || probs_dtype == MS_BF16 || probs_dtype == MS_FP16 || probs_dtype == MS_FP32,
+               MS_ERR_UNSUPPORTED, "ms_gmm_swiglu: probs dtype %d is not one of bf16/fp16/fp32", probs_dtype);
+    const SwigluOut extra{act, act_stride_row, probs, probs_dtype};
+    return gmm_impl(stream, x, x_stride0, x_stride1, weight, w_stride_group, w_stride0, w_stride1, y,
+                    y != nullptr ? y_stride_row : 2 * ffn, group_list, group_list_type, /*group_type=*/0, num_groups, m, k,
+                    2 * ffn, dtype, dtype, /*accumulate=*/0, workspace, workspace_bytes, nullptr, false, &extra);
 }
 
 extern "C" int ms_gmm_weight_list(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1,

@@ -41,9 +41,14 @@ struct GmmArgs {
     int64_t a_stride_row, a_stride_red;
     int64_t b_stride_red, b_stride_col;
     int64_t c_stride_row;
-    int cols;          // n
+    int cols;          // n (fused SwiGLU form: the number of activation columns, ffn = n / 2)
     int num_col_tiles;
     int a_vec_ok, b_vec_ok, c_vec_ok;
+    // fused SwiGLU form only (OUT_SWIGLU): second output and the per-row factor
+    void *act;                 // [rows, cols] activation output, same dtype
+    int64_t act_stride_row;
+    const void *probs;         // optional per-row probability
+    int probs_dtype;
 };
 
 struct TileCoord {
@@ -83,7 +88,7 @@ constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int kTileBytes = BM * BK * 2;                 // 32 KB per operand per stage
 constexpr int kLdsBytes16 = 4 * kTileBytes;             // A,B x 2 stages = 128 KB
 
-enum OutMode { OUT_SAME = 0, OUT_F32 = 1, ACC_F32 = 2 };
+enum OutMode { OUT_SAME = 0, OUT_F32 = 1, ACC_F32 = 2, OUT_SWIGLU = 3 };
 
 template <int DT>
 __device__ __forceinline__ f32x16 mfma16(v16 a, v16 b, f32x16 c) {

@@ -79,8 +79,12 @@ struct Operand {
 
     // outer0: first outer index of the tile; outer_last: clamp bound (RED: last valid outer index,
     // !RED: last valid start of an 8-wide chunk); wave_outer: this wavefront's first outer index in the tile.
+    // split (only for !RED, fused SwiGLU form): the second half of the tile's outer indices lies `split`
+    // elements further on in memory than the first half's continuation would (gate columns c0 .. c0+127 and
+    // up columns ffn+c0 .. ffn+c0+127 side by side in one tile: split = ffn - ROWS/2), with the clamp bound
+    // moved along by ffn.
     __device__ __forceinline__ void init(int64_t stride_outer, int64_t stride_red, int outer0, int outer_last,
-                                         int wave_outer) {
+                                         int wave_outer, int split = 0, int split_last = 0) {
         const int tid = threadIdx.x;
         const int lane = tid & 63;
         if constexpr (RED) {
@@ -99,8 +103,10 @@ struct Operand {
         } else {
             const int chunk = tid % CP;   // 16-byte chunk along the outer dim
             const int rrow = tid / CP;    // reduction row within one load of the workgroup
-            int outer = outer0 + chunk * 8;
-            outer = outer > outer_last ? outer_last : outer;
+            const bool second = chunk >= CP / 2;
+            int outer = outer0 + chunk * 8 + (second ? split : 0);
+            const int last = outer_last + (second ? split_last : 0);
+            outer = outer > last ? last : outer;
 #pragma unroll
             for (int i = 0; i < NL; ++i)
                 off[i] = static_cast<unsigned>((static_cast<int64_t>(i * RP + rrow) * stride_red + (outer - outer0)) * 2);
@@ -408,7 +414,9 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
 
     const int row0 = tc.e.row_begin + tc.row_tile * BM;   // all but the last row tile of a group are full
     const int row_end = tc.e.row_end;
-    const int col0 = tc.col_tile * BN;
+    constexpr bool SWIGLU = OUT == OUT_SWIGLU;
+    constexpr int HALF = BN / 2;                          // activation columns per tile in the fused form
+    const int col0 = tc.col_tile * (SWIGLU ? HALF : BN);  // fused: first activation (= gate) column
     const int col_end = p.cols;
     const int red_begin = tc.e.red_begin, red_end = tc.e.red_end;
 
@@ -426,7 +434,12 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
         Operand<A_RED, TBM> la;
         Operand<B_RED, BN> lb;
         la.init(p.a_stride_row, p.a_stride_red, row0, A_RED ? row_end - 1 : row_end - 8, wm * TM * 32);
+        if constexpr (SWIGLU) {
+        static_assert(!SWIGLU || !B_RED, "the fused SwiGLU form reads the weight along its columns");
+        lb.init(p.b_stride_col, p.b_stride_red, col0, col_end - 8, wn * TN * 32, col_end - HALF, col_end);
+    } else {
         lb.init(p.b_stride_col, p.b_stride_red, col0, B_RED ? col_end - 1 : col_end - 8, wn * TN * 32);
+    }
         // uniform base pointers of element (outer0, red_begin); advanced by one K step per iteration
         const char *a_ptr = static_cast<const char *>(p.a) +
                             (static_cast<int64_t>(row0) * p.a_stride_row + static_cast<int64_t>(red_begin) * p.a_stride_red) * 2;
@@ -542,7 +555,7 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
     //                                [col0 + wn*TN*32 + j*32 + 8*q + 4*(lane>>5) + e]
     const int64_t ldc = p.c_stride_row;
     constexpr int WR = TM * 32, WC = TN * 32;       // this wavefront's block of the tile
-    if constexpr (OUT == OUT_SAME) {
+    if constexpr (OUT == OUT_SAME || OUT == OUT_SWIGLU) {
         // 16-bit output: each wavefront stages its block in its own LDS region (row pitch WC*2 + 8 bytes:
         // conflict-free for the 8-byte column-slice writes and the row reads) and writes it out as 16 bytes
         // per lane, WC*2 contiguous bytes per row.
@@ -568,17 +581,55 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
         constexpr int LPR = WC / 8;            // lanes per row (8 columns = 16 bytes each)
         constexpr int RPP = 64 / LPR;          // rows per pass
         const int chunk = lane % LPR;
-        const int col = col0 + wn * WC + chunk * 8;
-        const bool col_ok = col < col_end;     // cols is a multiple of 8 on this path
-        uint16_t *cbase = static_cast<uint16_t *>(p.c) + tc.e.c_off + col;
+        // Fused form: the wavefronts of the first half of the tile's columns hold gate columns, their
+        // partners (same rows, other half) the matching up columns, ffn further on in the output row.
+        constexpr int GATE_WAVES = WAVES_N / 2;
+        const bool up_half = SWIGLU && wn >= GATE_WAVES;
+        const int acol = col0 + (SWIGLU ? wn % GATE_WAVES : wn) * WC + chunk * 8;   // activation column
+        const int col = SWIGLU ? acol + (up_half ? col_end : 0) : acol;
+        const bool col_ok = acol < col_end;    // cols is a multiple of 8 on this path
+        if (!SWIGLU || p.c != nullptr) {
+            uint16_t *cbase = static_cast<uint16_t *>(p.c) + tc.e.c_off + col;
 #pragma unroll 4
-        for (int pass = 0; pass < WR / RPP; ++pass) {
-            const int r = pass * RPP + lane / LPR;
-            const int row = row0 + wm * WR + r;
-            const uint2 lo = *reinterpret_cast<const uint2 *>(stg + r * SP + chunk * 16);
-            const uint2 hi2 = *reinterpret_cast<const uint2 *>(stg + r * SP + chunk * 16 + 8);
-            if (col_ok && row < row_end)
-                *reinterpret_cast<v16 *>(cbase + static_cast<int64_t>(row) * ldc) = v16{lo.x, lo.y, hi2.x, hi2.y};
+            for (int pass = 0; pass < WR / RPP; ++pass) {
+                const int r = pass * RPP + lane / LPR;
+                const int row = row0 + wm * WR + r;
+                const uint2 lo = *reinterpret_cast<const uint2 *>(stg + r * SP + chunk * 16);
+                const uint2 hi2 = *reinterpret_cast<const uint2 *>(stg + r * SP + chunk * 16 + 8);
+                if (col_ok && row < row_end)
+                    *reinterpret_cast<v16 *>(cbase + static_cast<int64_t>(row) * ldc) = v16{lo.x, lo.y, hi2.x, hi2.y};
+            }
+        }
+        if constexpr (SWIGLU) {
+            // act = silu(gate) * up * prob from the staged (already rounded) values, exactly what the
+            // stand-alone SwiGLU kernel computes from the stored fc1 output.  Each wavefront of a pair
+            // takes half of the rows.
+            using DTT = std::conditional_t<DT == MS_BF16, BF16, FP16>;
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_s_barrier();      // the partner's block is staged
+            const char *gstg = lds + (wm * WAVES_N + wn % GATE_WAVES) * kStagePerWave;
+            const char *ustg = gstg + GATE_WAVES * kStagePerWave;
+            const int rbase = up_half ? WR / 2 : 0;
+            uint16_t *abase = static_cast<uint16_t *>(p.act) + acol;
+#pragma unroll 4
+            for (int pass = 0; pass < WR / 2 / RPP; ++pass) {
+                const int r = rbase + pass * RPP + lane / LPR;
+                const int row = row0 + wm * WR + r;
+                uint16_t g[8], u[8], o[8];
+                *reinterpret_cast<uint2 *>(g) = *reinterpret_cast<const uint2 *>(gstg + r * SP + chunk * 16);
+                *reinterpret_cast<uint2 *>(g + 4) = *reinterpret_cast<const uint2 *>(gstg + r * SP + chunk * 16 + 8);
+                *reinterpret_cast<uint2 *>(u) = *reinterpret_cast<const uint2 *>(ustg + r * SP + chunk * 16);
+                *reinterpret_cast<uint2 *>(u + 4) = *reinterpret_cast<const uint2 *>(ustg + r * SP + chunk * 16 + 8);
+                if (col_ok && row < row_end) {
+                    const float pr = p.probs != nullptr ? load_scalar_as_float(p.probs, row, p.probs_dtype) : 1.f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float gf = DTT::to_float(g[e]);
+                        o[e] = DTT::from_float(gf * (1.f / (1.f + __expf(-gf))) * DTT::to_float(u[e]) * pr);
+                    }
+                    *reinterpret_cast<v16 *>(abase + static_cast<int64_t>(row) * p.act_stride_row) = *reinterpret_cast<v16 *>(o);
+                }
+            }
         }
     } else {
         const bool full_cols = col0 + BN <= col_end;
@@ -615,12 +666,15 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
 template <int DT, int OUT>
 int launch_fast(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red, unsigned grid) {
     const void *fn;
-    if (a_red && b_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, true, OUT>);
+    if constexpr (OUT == OUT_SWIGLU) {
+        MS_REQUIRE(a_red && !b_red, MS_ERR_UNSUPPORTED, "ms_gmm_swiglu: operand layout not supported");
+        fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, false, OUT>);
+    } else if (a_red && b_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, true, OUT>);
     else if (a_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, false, OUT>);
     else if (b_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, true, OUT>);
     else fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, false, OUT>);
     int lds_bytes = 2 * ((a_red ? kRedTileBytes : kOuterTileBytes) + (b_red ? kRedTileBytes : kOuterTileBytes));
-    if (OUT == OUT_SAME && lds_bytes < kStageBytes) lds_bytes = kStageBytes;
+    if ((OUT == OUT_SAME || OUT == OUT_SWIGLU) && lds_bytes < kStageBytes) lds_bytes = kStageBytes;
     if (!a_red && !b_red && lds_bytes < kRingBytes) lds_bytes = kRingBytes;   // use_ring<false, false>()
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "ms_gmm: hipFuncSetAttribute: %s", hipGetErrorString(e));
@@ -635,6 +689,10 @@ int launch_fast(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red,
 
 int launch_gmm16_fast(hipStream_t stream, const GmmArgs &args, int dtype, int out_mode, bool a_red, bool b_red,
                       unsigned grid) {
+    if (out_mode == OUT_SWIGLU) {
+        if (dtype == MS_BF16) return launch_fast<MS_BF16, OUT_SWIGLU>(stream, args, a_red, b_red, grid);
+        return launch_fast<MS_FP16, OUT_SWIGLU>(stream, args, a_red, b_red, grid);
+    }
     if (dtype == MS_BF16) {
         if (out_mode == OUT_SAME) return launch_fast<MS_BF16, OUT_SAME>(stream, args, a_red, b_red, grid);
         if (out_mode == OUT_F32) return launch_fast<MS_BF16, OUT_F32>(stream, args, a_red, b_red, grid);

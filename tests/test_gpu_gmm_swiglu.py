@@ -1,0 +1,103 @@
+"""GPU parity of the grouped matmul with the SwiGLU activation fused into its epilogue: against the CPU
+oracle (rel-L2 1e-2) and, bit for bit, against the two separate kernels it replaces."""
+import pytest
+import torch
+
+from conftest import rel_l2
+from oracle import moe_oracle as O
+
+import mindspeed_amd.ops as ops
+from mindspeed_amd.dispatcher import dispatch_mlp_combine, experts_computation
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+CASES = [
+    # counts, K, ffn, dtype, probs dtype (None = no probs), rows past the last offset
+    ([5, 0, 7, 3], 64, 128, torch.bfloat16, torch.float32, 0),
+    ([9, 0, 0, 7, 9, 6, 7, 4], 128, 200, torch.bfloat16, None, 0),          # ffn not a multiple of 128
+    ([130, 256, 1, 300, 64, 0, 200, 73], 256, 384, torch.bfloat16, torch.bfloat16, 5),   # 64-/128-row tails
+    ([300, 212], 72, 136, torch.float16, torch.float32, 0),
+    ([1024, 1000, 1048], 512, 1024, torch.bfloat16, torch.float32, 0),       # full tiles, many rounds
+    ([40], 8, 8, torch.bfloat16, torch.float32, 0),                          # smallest legal sizes
+]
+
+
+@pytest.mark.parametrize("counts,K,ffn,dtype,pdt,extra", CASES)
+def test_gmm_swiglu_forward_backward(counts, K, ffn, dtype, pdt, extra, device):
+    say("gmm_swiglu case", counts, K, ffn, dtype, pdt, extra)
+    E, M = len(counts), sum(counts) + extra
+    gen = torch.Generator().manual_seed(M + ffn)
+    x = torch.randn(M, K, generator=gen).to(dtype)
+    w = (torch.randn(E, K, 2 * ffn, generator=gen) * 0.1).to(dtype)
+    probs = None if pdt is None else (torch.rand(M, generator=gen) + 0.25).to(pdt)
+    g_act = torch.randn(M, ffn, generator=gen).to(dtype)
+    gl = torch.tensor(counts, dtype=torch.int64)
+
+    # the two separate kernels
+    xs = x.to(device).requires_grad_(True)
+    ws = w.to(device).requires_grad_(True)
+    ps = None if probs is None else probs.to(device).requires_grad_(True)
+    fc1 = ops.npu_gmm_v2(xs, ws, group_list=gl.to(device), group_type=0)
+    act_sep = ops.swiglu_with_probs(fc1, ps) if ps is not None else ops.fused_swiglu(fc1)
+    act_sep.backward(g_act.to(device))
+
+    # fused
+    xf = x.to(device).requires_grad_(True)
+    wf = w.to(device).requires_grad_(True)
+    pf = None if probs is None else probs.to(device).requires_grad_(True)
+    act = ops.gmm_swiglu(xf, wf, gl.to(device), pf)
+    act.backward(g_act.to(device))
+    torch.cuda.synchronize()
+    assert act.shape == (M, ffn) and act.dtype == dtype
+    assert torch.equal(act, act_sep)                       # same values, bit for bit
+    assert torch.equal(xf.grad, xs.grad) and torch.equal(wf.grad, ws.grad)
+    if probs is not None:
+        assert torch.equal(pf.grad, ps.grad)
+
+    # oracle (fc1 rounded to the storage dtype before the activation, as the op sequence does)
+    x64 = x.double().requires_grad_(True)
+    w64 = w.double().requires_grad_(True)
+    p64 = None if probs is None else probs.double().requires_grad_(True)
+    fc1_o = O.gmm(x64, w64, gl, group_type=0, group_list_type=1)
+    act_o = O.swiglu(fc1_o, p64)
+    act_o.backward(g_act.double())
+    assert rel_l2(act, act_o) <= 1e-2
+    assert rel_l2(xf.grad, x64.grad) <= 1e-2
+    assert rel_l2(wf.grad, w64.grad) <= 1e-2
+    if probs is not None:
+        assert rel_l2(pf.grad, p64.grad) <= 1e-2
+    if extra:
+        assert torch.count_nonzero(act[M - extra:]) == 0   # rows past the last offset
+
+
+def test_layer_uses_the_fused_kernel_and_matches_the_unfused_layer(device):
+    T, H, E, K, F = 300, 128, 8, 2, 256
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn(T, H, generator=gen).to(torch.bfloat16).to(device)
+    w1 = (torch.randn(E, H, 2 * F, generator=gen) * 0.05).to(torch.bfloat16).to(device)
+    w2 = (torch.randn(E, F, H, generator=gen) * 0.05).to(torch.bfloat16).to(device)
+    p, idx = O.route_topk(torch.randn(T, E, generator=gen), K)
+    p, idx = p.to(torch.bfloat16).to(device), idx.to(device)
+    from mindspeed_amd import flop_counter
+    with flop_counter.record(timing=False) as rec:
+        out = dispatch_mlp_combine(x, idx, p, (w1, w2))
+    names = [c[0] for c in rec.calls]
+    assert "swiglu" not in names and names.count("gmm_fwd") == 2      # activation came out of the first matmul
+    perm, rmap, _, counts = ops.moe_token_permute_with_aux(x, idx, num_experts=E)
+    ref = ops.npu_moe_token_unpermute(experts_computation(perm, counts, w1, w2, fuse_activation=False), rmap, p)
+    assert torch.equal(out, ref)
+
+
+def test_unsupported_layout_is_reported(device):
+    x = torch.randn(16, 12, device=device).to(torch.bfloat16)            # K not a multiple of 8
+    w = torch.randn(2, 12, 32, device=device).to(torch.bfloat16)
+    gl = torch.tensor([8, 8], dtype=torch.int64, device=device)
+    with pytest.raises(Exception, match="vector-access"):
+        ops.gmm_swiglu(x, w, gl)
+    with pytest.raises(TypeError):
+        ops.gmm_swiglu(x.float(), w.float(), gl)
