@@ -203,6 +203,25 @@ int ms_gmm_swiglu(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t 
                   int probs_dtype, const int64_t *group_list, int group_list_type, int64_t num_groups,
                   int64_t m, int64_t k, int64_t ffn, int dtype, void *workspace, size_t workspace_bytes);
 
+/* Backward counterpart: dact = dy @ W2^T (the dX product of the second grouped matmul) with the
+ * SwiGLU backward of mindspeed/ops/csrc/atb/swiglu.cpp:96-126 (and the probability factor of
+ * experts.py:41-44) fused into its epilogue, so dact is never written:
+ *   d_fc1[r, c]       = dact[r, c] * probs[r] * up   * sig * (1 + gate * (1 - sig))
+ *   d_fc1[r, ffn + c] = dact[r, c] * probs[r] * gate * sig            (sig = sigmoid(gate))
+ *   grad_probs[r]     = sum_c dact[r, c] * gate * sig * up            (fp32; summed per 64 columns
+ *                       in the epilogue, then over the row by a second small kernel)
+ * with gate = fc1[r, c], up = fc1[r, ffn + c] and dact rounded to dtype first, i.e. the values
+ * ms_gmm followed by ms_swiglu_grad produce.  dy [m, k]; weight is the transposed view of
+ * W2 [num_groups, ffn, k] (w_stride0 = 1 along k, w_stride1 = k along ffn); fc1 / d_fc1 [m, 2*ffn];
+ * probs / grad_probs optional together.  Same layout conditions as ms_gmm_swiglu. */
+int ms_gmm_swiglu_grad_workspace_size(int64_t num_groups, int64_t m, int64_t ffn, size_t *bytes);
+int ms_gmm_swiglu_grad(ms_stream_t stream, const void *dy, int64_t dy_stride0, int64_t dy_stride1,
+                       const void *weight, int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1,
+                       const void *fc1, int64_t fc1_stride_row, const void *probs, int probs_dtype,
+                       void *d_fc1, int64_t d_fc1_stride_row, void *grad_probs,
+                       const int64_t *group_list, int group_list_type, int64_t num_groups, int64_t m,
+                       int64_t k, int64_t ffn, int dtype, void *workspace, size_t workspace_bytes);
+
 /* The same product (group_type 0 only) with one separately allocated weight matrix per group —
  * the form torch_npu.npu_grouped_matmul([x], [w_0 .. w_{E-1}], ...) takes from
  * mindspeed/te/pytorch/module/grouped_linear.py:61-69,85-93 (per-expert parameters

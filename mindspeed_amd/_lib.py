@@ -46,6 +46,9 @@ _SIGNATURES = {
                _i64, _i64, _i64, _i64, _int, _int, _int, _c_void_p, _size_t],
     "ms_gmm_swiglu": [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _i64, _i64, _i64, _c_void_p, _i64, _c_void_p, _i64,
                       _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _int, _c_void_p, _size_t],
+    "ms_gmm_swiglu_grad_workspace_size": [_i64, _i64, _i64, ctypes.POINTER(_size_t)],
+    "ms_gmm_swiglu_grad": [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _i64, _i64, _i64, _c_void_p, _i64, _c_void_p, _int,
+                           _c_void_p, _i64, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _i64, _int, _c_void_p, _size_t],
     "ms_gmm_weight_list": [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _i64, _i64, _c_void_p, _i64, _c_void_p, _int,
                            _i64, _i64, _i64, _i64, _int, _int, _c_void_p, _size_t],
     "ms_swiglu": [_c_void_p, _c_void_p, _c_void_p, _int, _i64, _i64, _int, _c_void_p],

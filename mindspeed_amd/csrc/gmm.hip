@@ -498,13 +498,35 @@ struct SwigluOut {
     const void *probs;
     int probs_dtype;
 };
+// Inputs of the fused SwiGLU backward form (the product is dact [m, ffn]; what is written is d_fc1 [m, 2*ffn]).
+struct SwigluGradIn {
+    const void *fc1;
+    int64_t fc1_stride_row;
+    const void *probs;
+    int probs_dtype;
+    float *partials;
+    int partials_per_row;
+};
+
+// grad_probs[r] = sum of the row's partial sums, in the probabilities' dtype.  One wavefront per row.
+__global__ __launch_bounds__(256) void swiglu_grad_probs_kernel(const float *__restrict__ partials, int per_row, int rows,
+                                                                void *__restrict__ grad_probs, int probs_dtype) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= rows) return;
+    float s = 0.f;
+    for (int i = lane; i < per_row; i += 64) s += partials[static_cast<int64_t>(row) * per_row + i];
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) s += __shfl_down(s, d, 64);
+    if (lane == 0) store_float_as(grad_probs, row, probs_dtype, s);
+}
 
 static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64_t x_stride1, const void *weight,
                     int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1, void *y, int64_t y_stride_row,
                     const int64_t *group_list, int group_list_type, int group_type, int64_t num_groups, int64_t m,
                     int64_t k, int64_t n, int dtype, int out_dtype, int accumulate, void *workspace,
                     size_t workspace_bytes, const WeightOffsets *weight_offsets, bool all_weights_aligned16,
-                    const SwigluOut *swiglu = nullptr) {
+                    const SwigluOut *swiglu = nullptr, const SwigluGradIn *swiglu_grad = nullptr) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED, "ms_gmm: bad dtype %d", dtype);
     MS_REQUIRE(out_dtype == dtype || out_dtype == MS_FP32, MS_ERR_UNSUPPORTED,
@@ -616,6 +638,16 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     if (swiglu != nullptr)   // 16-byte row stores of both outputs, whole 8-column chunks in each half
         args.c_vec_ok = aligned16(y) && y_stride_row % 8 == 0 && aligned16(swiglu->act) &&
                         swiglu->act_stride_row % 8 == 0 && (n / 2) % 8 == 0;
+    if (swiglu_grad != nullptr) {
+        args.c_vec_ok = aligned16(y) && y_stride_row % 8 == 0 && aligned16(swiglu_grad->fc1) &&
+                        swiglu_grad->fc1_stride_row % 8 == 0 && n % 8 == 0;
+        args.fc1 = swiglu_grad->fc1;
+        args.fc1_stride_row = swiglu_grad->fc1_stride_row;
+        args.probs = swiglu_grad->probs;
+        args.probs_dtype = swiglu_grad->probs_dtype;
+        args.partials = swiglu_grad->partials;
+        args.partials_per_row = swiglu_grad->partials_per_row;
+    }
     // A stride of 1 in a dim of extent 1 may come with an arbitrary other stride.
     const bool a_is_red = use_a_red || !a_row;
     const bool b_is_red = use_b_red || !b_col;
@@ -642,6 +674,13 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
                    "along k, weight contiguous along its columns, k and ffn multiples of 8)");
         if (int rc = schedule(1)) return rc;
         return launch_gmm16_fast(stream, args, dtype, OUT_SWIGLU, true, false, grid);
+    }
+    if (swiglu_grad != nullptr) {
+        MS_REQUIRE(fast && a_is_red && b_is_red, MS_ERR_UNSUPPORTED,
+                   "ms_gmm_swiglu_grad: needs the vector-access layout (16-byte aligned operands and outputs, dy and the "
+                   "transposed weight view contiguous along k, k and ffn multiples of 8)");
+        if (int rc = schedule(1)) return rc;
+        return launch_gmm16_fast(stream, args, dtype, OUT_SWIGLU_GRAD, true, true, grid);
     }
     if (int rc = schedule(fast ? 1 : 0)) return rc;
     if (fast) return launch_gmm16_fast(stream, args, dtype, out, a_is_red, b_is_red, grid);
@@ -681,6 +720,59 @@ extern "C" int ms_gmm_swiglu(ms_stream_t stream, const void *x, int64_t x_stride
     return gmm_impl(stream, x, x_stride0, x_stride1, weight, w_stride_group, w_stride0, w_stride1, y,
                     y != nullptr ? y_stride_row : 2 * ffn, group_list, group_list_type, /*group_type=*/0, num_groups, m, k,
                     2 * ffn, dtype, dtype, /*accumulate=*/0, workspace, workspace_bytes, nullptr, false, &extra);
+}
+
+namespace {
+int64_t swiglu_partials_per_row(int64_t ffn) { return (ffn + 63) / 64; }
+size_t swiglu_grad_partials_pos(int64_t num_groups) { return (workspace_need(num_groups) + 255) & ~static_cast<size_t>(255); }
+}  // namespace
+
+extern "C" int ms_gmm_swiglu_grad_workspace_size(int64_t num_groups, int64_t m, int64_t ffn, size_t *bytes) {
+    MS_REQUIRE(bytes != nullptr, MS_ERR_INVALID_ARGUMENT, "ms_gmm_swiglu_grad_workspace_size: bytes is NULL");
+    MS_REQUIRE(num_groups >= 1 && num_groups <= kMaxGroups && m >= 0 && ffn >= 0, MS_ERR_INVALID_ARGUMENT,
+               "ms_gmm_swiglu_grad_workspace_size: bad sizes");
+    *bytes = swiglu_grad_partials_pos(num_groups) +
+             ((static_cast<size_t>(m) * swiglu_partials_per_row(ffn) * sizeof(float) + 255) & ~static_cast<size_t>(255));
+    return MS_OK;
+}
+
+extern "C" int ms_gmm_swiglu_grad(ms_stream_t stream, const void *dy, int64_t dy_stride0, int64_t dy_stride1,
+                                  const void *weight, int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1,
+                                  const void *fc1, int64_t fc1_stride_row, const void *probs, int probs_dtype,
+                                  void *d_fc1, int64_t d_fc1_stride_row, void *grad_probs, const int64_t *group_list,
+                                  int group_list_type, int64_t num_groups, int64_t m, int64_t k, int64_t ffn, int dtype,
+                                  void *workspace, size_t workspace_bytes) {
+    const char *fn = "ms_gmm_swiglu_grad";
+    MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16, MS_ERR_UNSUPPORTED, "%s: dtype must be bf16 or fp16", fn);
+    MS_REQUIRE(ffn >= 0 && ffn < (1ll << 30) && m >= 0, MS_ERR_INVALID_ARGUMENT, "%s: bad sizes", fn);
+    MS_REQUIRE(num_groups >= 1 && num_groups <= kMaxGroups, MS_ERR_UNSUPPORTED, "%s: num_groups %lld outside [1, %d]", fn,
+               (long long)num_groups, kMaxGroups);
+    MS_REQUIRE((probs == nullptr) == (grad_probs == nullptr), MS_ERR_INVALID_ARGUMENT,
+               "%s: probs and grad_probs must be given together", fn);
+    MS_REQUIRE(probs == nullptr || probs_dtype == MS_BF16 || probs_dtype == MS_FP16 || probs_dtype == MS_FP32,
+               MS_ERR_UNSUPPORTED, "%s: probs dtype %d is not one of bf16/fp16/fp32", fn, probs_dtype);
+    if (m == 0 || ffn == 0) return MS_OK;
+    MS_REQUIRE(fc1 != nullptr && d_fc1 != nullptr, MS_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", fn);
+    MS_REQUIRE(fc1_stride_row >= 2 * ffn && d_fc1_stride_row >= 2 * ffn, MS_ERR_INVALID_ARGUMENT,
+               "%s: fc1 / d_fc1 row strides must be at least 2*ffn", fn);
+    size_t need = 0;
+    if (int rc = ms_gmm_swiglu_grad_workspace_size(num_groups, m, ffn, &need)) return rc;
+    MS_REQUIRE(workspace != nullptr && workspace_bytes >= need, MS_ERR_WORKSPACE_TOO_SMALL, "%s: workspace %zu < %zu bytes",
+               fn, workspace_bytes, need);
+    const int per_row = static_cast<int>(swiglu_partials_per_row(ffn));
+    float *partials = grad_probs != nullptr
+        ? reinterpret_cast<float *>(static_cast<char *>(workspace) + swiglu_grad_partials_pos(num_groups)) : nullptr;
+    const SwigluGradIn extra{fc1, fc1_stride_row, probs, probs_dtype, partials, per_row};
+    if (int rc = gmm_impl(stream, dy, dy_stride0, dy_stride1, weight, w_stride_group, w_stride0, w_stride1, d_fc1,
+                          d_fc1_stride_row, group_list, group_list_type, /*group_type=*/0, num_groups, m, k, ffn, dtype,
+                          dtype, /*accumulate=*/0, workspace, workspace_bytes, nullptr, false, nullptr, &extra))
+        return rc;
+    if (grad_probs != nullptr) {
+        hipLaunchKernelGGL(swiglu_grad_probs_kernel, dim3(static_cast<unsigned>(ceil_div(m, 4))), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), partials, per_row, static_cast<int>(m), grad_probs, probs_dtype);
+        MS_CHECK_LAUNCH("swiglu_grad_probs_kernel");
+    }
+    return MS_OK;
 }
 
 extern "C" int ms_gmm_weight_list(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1,

@@ -49,6 +49,11 @@ struct GmmArgs {
     int64_t act_stride_row;
     const void *probs;         // optional per-row probability
     int probs_dtype;
+    // fused SwiGLU backward form only (OUT_SWIGLU_GRAD): c is d_fc1 [rows, 2*cols]
+    const void *fc1;           // [rows, 2*cols] saved output of the first matmul (gate | up)
+    int64_t fc1_stride_row;
+    float *partials;           // [rows, partials_per_row] row sums of dact * silu(gate) * up per 64 columns, or NULL
+    int partials_per_row;
 };
 
 struct TileCoord {
@@ -88,7 +93,7 @@ constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int kTileBytes = BM * BK * 2;                 // 32 KB per operand per stage
 constexpr int kLdsBytes16 = 4 * kTileBytes;             // A,B x 2 stages = 128 KB
 
-enum OutMode { OUT_SAME = 0, OUT_F32 = 1, ACC_F32 = 2, OUT_SWIGLU = 3 };
+enum OutMode { OUT_SAME = 0, OUT_F32 = 1, ACC_F32 = 2, OUT_SWIGLU = 3, OUT_SWIGLU_GRAD = 4 };
 
 template <int DT>
 __device__ __forceinline__ f32x16 mfma16(v16 a, v16 b, f32x16 c) {

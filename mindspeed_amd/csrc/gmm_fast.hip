@@ -555,7 +555,7 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
     //                                [col0 + wn*TN*32 + j*32 + 8*q + 4*(lane>>5) + e]
     const int64_t ldc = p.c_stride_row;
     constexpr int WR = TM * 32, WC = TN * 32;       // this wavefront's block of the tile
-    if constexpr (OUT == OUT_SAME || OUT == OUT_SWIGLU) {
+    if constexpr (OUT == OUT_SAME || OUT == OUT_SWIGLU || OUT == OUT_SWIGLU_GRAD) {
         // 16-bit output: each wavefront stages its block in its own LDS region (row pitch WC*2 + 8 bytes:
         // conflict-free for the 8-byte column-slice writes and the row reads) and writes it out as 16 bytes
         // per lane, WC*2 contiguous bytes per row.
@@ -588,7 +588,51 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
         const int acol = col0 + (SWIGLU ? wn % GATE_WAVES : wn) * WC + chunk * 8;   // activation column
         const int col = SWIGLU ? acol + (up_half ? col_end : 0) : acol;
         const bool col_ok = acol < col_end;    // cols is a multiple of 8 on this path
-        if (!SWIGLU || p.c != nullptr) {
+        if constexpr (OUT == OUT_SWIGLU_GRAD) {
+            // The staged block is dact = dY @ W2^T (rounded, as the stand-alone matmul would store it); what is
+            // written is d_fc1 = SwiGLU backward of it on the saved fc1 output, the same arithmetic as the
+            // stand-alone kernel, and per 64 columns the row sums that make up the probabilities' gradient.
+            using DTT = std::conditional_t<DT == MS_BF16, BF16, FP16>;
+            const uint16_t *fbase = static_cast<const uint16_t *>(p.fc1) + acol;
+            uint16_t *dbase = static_cast<uint16_t *>(p.c) + acol;
+#pragma unroll 2
+            for (int pass = 0; pass < WR / RPP; ++pass) {
+                const int r = pass * RPP + lane / LPR;
+                const int row = row0 + wm * WR + r;
+                const bool ok = col_ok && row < row_end;
+                uint16_t d[8], g[8], u[8], og[8], ou[8];
+                *reinterpret_cast<uint2 *>(d) = *reinterpret_cast<const uint2 *>(stg + r * SP + chunk * 16);
+                *reinterpret_cast<uint2 *>(d + 4) = *reinterpret_cast<const uint2 *>(stg + r * SP + chunk * 16 + 8);
+                float dot = 0.f;
+                if (ok) {
+                    const uint16_t *fg = fbase + static_cast<int64_t>(row) * p.fc1_stride_row;
+                    *reinterpret_cast<v16 *>(g) = *reinterpret_cast<const v16 *>(fg);
+                    *reinterpret_cast<v16 *>(u) = *reinterpret_cast<const v16 *>(fg + col_end);
+                    const float pr = p.probs != nullptr ? load_scalar_as_float(p.probs, row, p.probs_dtype) : 1.f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float gf = DTT::to_float(g[e]), uf = DTT::to_float(u[e]), df = DTT::to_float(d[e]);
+                        const float sig = 1.f / (1.f + __expf(-gf));
+                        const float act = gf * sig;
+                        dot = fmaf(df, act * uf, dot);
+                        const float dp = df * pr;
+                        og[e] = DTT::from_float(dp * uf * (sig * (1.f + gf * (1.f - sig))));
+                        ou[e] = DTT::from_float(dp * act);
+                    }
+                    uint16_t *dg = dbase + static_cast<int64_t>(row) * ldc;
+                    *reinterpret_cast<v16 *>(dg) = *reinterpret_cast<v16 *>(og);
+                    *reinterpret_cast<v16 *>(dg + col_end) = *reinterpret_cast<v16 *>(ou);
+                }
+                if (p.partials != nullptr) {
+                    // 8 lanes = 64 columns: one partial sum per row and 64-column block
+                    dot += __shfl_xor(dot, 1, 64);
+                    dot += __shfl_xor(dot, 2, 64);
+                    dot += __shfl_xor(dot, 4, 64);
+                    if ((chunk & 7) == 0 && ok)
+                        p.partials[static_cast<int64_t>(row) * p.partials_per_row + (acol >> 6)] = dot;
+                }
+            }
+        } else if (!SWIGLU || p.c != nullptr) {
             uint16_t *cbase = static_cast<uint16_t *>(p.c) + tc.e.c_off + col;
 #pragma unroll 4
             for (int pass = 0; pass < WR / RPP; ++pass) {
@@ -669,12 +713,15 @@ int launch_fast(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red,
     if constexpr (OUT == OUT_SWIGLU) {
         MS_REQUIRE(a_red && !b_red, MS_ERR_UNSUPPORTED, "ms_gmm_swiglu: operand layout not supported");
         fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, false, OUT>);
+    } else if constexpr (OUT == OUT_SWIGLU_GRAD) {
+        MS_REQUIRE(a_red && b_red, MS_ERR_UNSUPPORTED, "ms_gmm_swiglu_grad: operand layout not supported");
+        fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, true, OUT>);
     } else if (a_red && b_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, true, OUT>);
     else if (a_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, false, OUT>);
     else if (b_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, true, OUT>);
     else fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, false, OUT>);
     int lds_bytes = 2 * ((a_red ? kRedTileBytes : kOuterTileBytes) + (b_red ? kRedTileBytes : kOuterTileBytes));
-    if ((OUT == OUT_SAME || OUT == OUT_SWIGLU) && lds_bytes < kStageBytes) lds_bytes = kStageBytes;
+    if ((OUT == OUT_SAME || OUT == OUT_SWIGLU || OUT == OUT_SWIGLU_GRAD) && lds_bytes < kStageBytes) lds_bytes = kStageBytes;
     if (!a_red && !b_red && lds_bytes < kRingBytes) lds_bytes = kRingBytes;   // use_ring<false, false>()
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "ms_gmm: hipFuncSetAttribute: %s", hipGetErrorString(e));
@@ -692,6 +739,10 @@ int launch_gmm16_fast(hipStream_t stream, const GmmArgs &args, int dtype, int ou
     if (out_mode == OUT_SWIGLU) {
         if (dtype == MS_BF16) return launch_fast<MS_BF16, OUT_SWIGLU>(stream, args, a_red, b_red, grid);
         return launch_fast<MS_FP16, OUT_SWIGLU>(stream, args, a_red, b_red, grid);
+    }
+    if (out_mode == OUT_SWIGLU_GRAD) {
+        if (dtype == MS_BF16) return launch_fast<MS_BF16, OUT_SWIGLU_GRAD>(stream, args, a_red, b_red, grid);
+        return launch_fast<MS_FP16, OUT_SWIGLU_GRAD>(stream, args, a_red, b_red, grid);
     }
     if (dtype == MS_BF16) {
         if (out_mode == OUT_SAME) return launch_fast<MS_BF16, OUT_SAME>(stream, args, a_red, b_red, grid);

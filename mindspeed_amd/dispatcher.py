@@ -10,29 +10,32 @@ from __future__ import annotations
 
 import torch
 
-from .ops import (fused_swiglu, gmm_swiglu, moe_token_permute_with_aux, npu_gmm_v2, npu_moe_token_unpermute)
+from .ops import (fused_swiglu, grouped_mlp, moe_token_permute_with_aux, npu_gmm_v2, npu_moe_token_unpermute)
 
 __all__ = ["experts_computation", "dispatch_mlp_combine"]
 
 
-def _fusable(hidden_states, gate_up_weights):
-    """Whether the fused matmul + SwiGLU kernel takes these operands (16-bit, vector-access layout)."""
+def _fusable(hidden_states, gate_up_weights, down_weights):
+    """Whether the fused matmul + SwiGLU kernels take these operands (16-bit, vector-access layout)."""
     ffn = gate_up_weights.size(-1) // 2
     return (hidden_states.dtype in (torch.bfloat16, torch.float16) and gate_up_weights.dim() == 3
+            and down_weights.dim() == 3 and down_weights.dtype == hidden_states.dtype
             and hidden_states.size(-1) % 8 == 0 and ffn % 8 == 0 and gate_up_weights.size(-1) % 2 == 0
-            and hidden_states.data_ptr() % 16 == 0 and gate_up_weights.data_ptr() % 16 == 0)
+            and down_weights.size(-1) % 8 == 0 and down_weights.size(1) == ffn
+            and hidden_states.data_ptr() % 16 == 0 and gate_up_weights.data_ptr() % 16 == 0
+            and down_weights.data_ptr() % 16 == 0)
 
 
 def experts_computation(hidden_states, split_list, gate_up_weights, down_weights, fuse_activation=True):
     """``gmm -> silu(gate) * up -> gmm`` (dispatcher.py:93-104); ``split_list`` = rows per expert.
 
-    With ``fuse_activation`` the activation comes out of the first grouped matmul's epilogue (same values as the
-    separate kernel's) whenever the operands allow it."""
-    if fuse_activation and _fusable(hidden_states, gate_up_weights):
-        act = gmm_swiglu(hidden_states, gate_up_weights, split_list)
-    else:
-        fc1 = npu_gmm_v2(hidden_states, gate_up_weights, group_list=split_list, group_type=0)
-        act = fused_swiglu(fc1)
+    With ``fuse_activation`` the activation comes out of the first grouped matmul's epilogue and its backward
+    rides on the epilogue of the second matmul's dX product (same values as the separate kernels') whenever
+    the operands allow it."""
+    if fuse_activation and _fusable(hidden_states, gate_up_weights, down_weights):
+        return grouped_mlp(hidden_states, gate_up_weights, down_weights, split_list)
+    fc1 = npu_gmm_v2(hidden_states, gate_up_weights, group_list=split_list, group_type=0)
+    act = fused_swiglu(fc1)
     return npu_gmm_v2(act, down_weights, group_list=split_list, group_type=0)
 
 

@@ -8,4 +8,4 @@ from .sort_chunks import sort_chunks_by_idxs  # noqa: F401
 from .moe_permute_mask_map import MoePermuteMaskMap, MoeUnpermuteMaskMap  # noqa: F401
 from .grouped_matmul import _GroupedMatmul, fused_grouped_matmul  # noqa: F401
 from .te_grouped_linear import MindSpeedTEGroupedLinearGMM, MindSpeedTEGroupedLinear  # noqa: F401
-from .gmm_swiglu import gmm_swiglu, GmmSwigluFunction  # noqa: F401
+from .gmm_swiglu import gmm_swiglu, GmmSwigluFunction, grouped_mlp, GroupedMLPFunction  # noqa: F401

@@ -101,3 +101,61 @@ def test_unsupported_layout_is_reported(device):
         ops.gmm_swiglu(x, w, gl)
     with pytest.raises(TypeError):
         ops.gmm_swiglu(x.float(), w.float(), gl)
+
+
+MLP_CASES = [
+    # counts, K (hidden), ffn, dtype, probs dtype, rows past the last offset
+    ([5, 0, 7, 3], 64, 128, torch.bfloat16, torch.float32, 0),
+    ([9, 0, 0, 7, 9, 6, 7, 4], 128, 200, torch.bfloat16, None, 0),
+    ([130, 256, 1, 300, 64, 0, 200, 73], 256, 384, torch.bfloat16, torch.bfloat16, 5),
+    ([300, 212], 72, 136, torch.float16, torch.float32, 0),
+    ([700, 1000, 348], 512, 1024, torch.bfloat16, torch.float32, 0),
+]
+
+
+@pytest.mark.parametrize("counts,K,ffn,dtype,pdt,extra", MLP_CASES)
+@pytest.mark.parametrize("recompute", [False, True])
+def test_grouped_mlp_forward_backward(counts, K, ffn, dtype, pdt, extra, recompute, device):
+    say("grouped_mlp case", counts, K, ffn, dtype, pdt, extra, recompute)
+    E, M = len(counts), sum(counts) + extra
+    gen = torch.Generator().manual_seed(M + ffn + 1)
+    x = torch.randn(M, K, generator=gen).to(dtype)
+    w1 = (torch.randn(E, K, 2 * ffn, generator=gen) * 0.1).to(dtype)
+    w2 = (torch.randn(E, ffn, K, generator=gen) * 0.1).to(dtype)
+    probs = None if pdt is None else (torch.rand(M, generator=gen) + 0.25).to(pdt)
+    gy = torch.randn(M, K, generator=gen).to(dtype)
+    gl = torch.tensor(counts, dtype=torch.int64)
+
+    def leaves():
+        out = [t.to(device).requires_grad_(True) for t in (x, w1, w2)]
+        out.append(None if probs is None else probs.to(device).requires_grad_(True))
+        return out
+
+    # the separate kernels
+    xs, w1s, w2s, ps = leaves()
+    fc1 = ops.npu_gmm_v2(xs, w1s, group_list=gl.to(device), group_type=0)
+    act = ops.swiglu_with_probs(fc1, ps) if ps is not None else ops.fused_swiglu(fc1)
+    out_sep = ops.npu_gmm_v2(act, w2s, group_list=gl.to(device), group_type=0)
+    out_sep.backward(gy.to(device))
+
+    xf, w1f, w2f, pf = leaves()
+    out = ops.grouped_mlp(xf, w1f, w2f, gl.to(device), pf, recompute_activation=recompute)
+    out.backward(gy.to(device))
+    torch.cuda.synchronize()
+    assert torch.equal(out, out_sep)
+    assert torch.equal(xf.grad, xs.grad)                   # d_fc1 is bit-identical, so everything behind it is
+    assert torch.equal(w1f.grad, w1s.grad) and torch.equal(w2f.grad, w2s.grad)
+    if probs is not None:
+        # same terms, summed per 64 columns and then over the row instead of in one pass
+        assert rel_l2(pf.grad, ps.grad) <= (1e-5 if pdt == torch.float32 else 1e-2)
+
+    x64, w164, w264 = (t.double().requires_grad_(True) for t in (x, w1, w2))
+    p64 = None if probs is None else probs.double().requires_grad_(True)
+    fc1_o = O.gmm(x64, w164, gl, group_type=0, group_list_type=1)
+    out_o = O.gmm(O.swiglu(fc1_o, p64), w264, gl, group_type=0, group_list_type=1)
+    out_o.backward(gy.double())
+    assert rel_l2(out, out_o) <= 1e-2
+    assert rel_l2(xf.grad, x64.grad) <= 1e-2
+    assert rel_l2(w1f.grad, w164.grad) <= 1e-2 and rel_l2(w2f.grad, w264.grad) <= 1e-2
+    if probs is not None:
+        assert rel_l2(pf.grad, p64.grad) <= 1e-2
