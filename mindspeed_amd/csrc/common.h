@@ -14,13 +14,8 @@ namespace ms {
 typedef unsigned int v16 __attribute__((ext_vector_type(4)));
 
 // Streaming (non-temporal) access for data that is touched once.
-#ifdef EXP_PLAIN_ACCESS
-#define MS_NT_LOAD(p) (*(p))
-#define MS_NT_STORE(v, p) (*(p) = (v))
-#else
 #define MS_NT_LOAD(p) __builtin_nontemporal_load(p)
 #define MS_NT_STORE(v, p) __builtin_nontemporal_store((v), (p))
-#endif
 
 // ---- host-side error plumbing ------------------------------------------------
 void set_error(const char *fmt, ...);

@@ -115,6 +115,8 @@ class MoePermuteMaskMap(torch.autograd.Function):
                 ) -> Tuple[torch.Tensor, Optional[torch.Tensor], torch.Tensor]:
         if tokens.dim() != 2:
             raise RuntimeError(f"The dims of input tokens should be 2 dimensional, but got {tokens.dim()}-dimensional.")
+        if routing_map is not None and routing_map.dtype != torch.bool:
+            raise TypeError(f"routing_map dtype [{routing_map.dtype}] is invalid, should be bool")
         _lib.require_device(tokens, "tokens")
         _check_map(routing_map, tokens.size(0))
         lib = _lib.load()
@@ -190,6 +192,8 @@ class MoeUnpermuteMaskMap(torch.autograd.Function):
         if permuted_tokens.dim() != 2:
             raise RuntimeError("The dims of input permuted_tokens should be 2 dimensional, "
                                f"but got {permuted_tokens.dim()}-dimensional.")
+        if routing_map is None:
+            raise ValueError("routing_map is required")
         _lib.require_device(permuted_tokens, "permuted_tokens")
         if sorted_indices.numel() != permuted_tokens.size(0):   # unpermute_without_activation.py:35-36
             raise AssertionError("sorted_indices must have one entry per permuted row")

@@ -114,3 +114,37 @@ def test_groupmatmul_add_checks():
         ops.npu_groupmatmul_add_fp32(x, dy, torch.tensor([4, 8]), torch.zeros(32, 4, dtype=torch.bfloat16))
     with pytest.raises(ValueError, match="elements"):
         ops.npu_groupmatmul_add_fp32(x, dy, torch.tensor([4, 8]), torch.zeros(31, 4))
+
+
+def test_routing_map_and_module_api_surface():
+    from mindspeed_amd.ops import moe_permute_mask_map as M
+    # mindspeed/core/fusions/fused_moe_permute.py:50-57,69-77
+    assert list(inspect.signature(M.permute).parameters) == [
+        "tokens", "routing_map", "probs", "num_out_tokens", "fused", "drop_and_pad"]
+    assert list(inspect.signature(M.unpermute).parameters) == [
+        "permuted_tokens", "sorted_indices", "restore_shape", "probs", "routing_map", "fused", "drop_and_pad"]
+    # mindspeed/ops/grouped_matmul.py:81
+    assert list(inspect.signature(ops.fused_grouped_matmul).parameters) == ["inputs", "m_split", "weights"]
+    x = torch.randn(8, 16, dtype=torch.bfloat16)
+    rmap = torch.ones(8, 2, dtype=torch.bool)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        M.permute(x, rmap)
+    with pytest.raises(TypeError, match="should be bool"):
+        M.permute(x, rmap.to(torch.int8))
+    with pytest.raises(ValueError, match="routing_map is required"):
+        M.unpermute(x, torch.zeros(8, dtype=torch.int64), x.shape)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.fused_grouped_matmul(x, [4, 4], torch.randn(2, 16, 4, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.MindSpeedTEGroupedLinear(2, 16, 4, params_dtype=torch.bfloat16)(x, [4, 4])
+    with pytest.raises(ValueError, match="bias"):
+        ops._GroupedMatmul.apply(x, torch.randn(2, 16, 4, dtype=torch.bfloat16), torch.zeros(4), [4, 4], 1)
+
+
+def test_fused_mlp_argument_checks():
+    x = torch.randn(8, 16, dtype=torch.bfloat16)
+    w1 = torch.randn(2, 16, 8, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.gmm_swiglu(x, w1, torch.tensor([4, 4]))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.grouped_mlp(x, w1, torch.randn(2, 4, 16, dtype=torch.bfloat16), torch.tensor([4, 4]))
