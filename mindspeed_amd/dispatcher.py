@@ -26,12 +26,13 @@ def _fusable(hidden_states, gate_up_weights, down_weights):
             and down_weights.data_ptr() % 16 == 0)
 
 
-def experts_computation(hidden_states, split_list, gate_up_weights, down_weights, fuse_activation=True):
+def experts_computation(hidden_states, split_list, gate_up_weights, down_weights, fuse_activation=False):
     """``gmm -> silu(gate) * up -> gmm`` (dispatcher.py:93-104); ``split_list`` = rows per expert.
 
-    With ``fuse_activation`` the activation comes out of the first grouped matmul's epilogue and its backward
-    rides on the epilogue of the second matmul's dX product (same values as the separate kernels') whenever
-    the operands allow it."""
+    The default is the reference's op sequence, one kernel per op.  With ``fuse_activation`` the activation
+    comes out of the first grouped matmul's epilogue and its backward rides on the epilogue of the second
+    matmul's dX product (same values as the separate kernels', same step time, one buffer and two launches
+    fewer) whenever the operands allow it."""
     if fuse_activation and _fusable(hidden_states, gate_up_weights, down_weights):
         return grouped_mlp(hidden_states, gate_up_weights, down_weights, split_list)
     fc1 = npu_gmm_v2(hidden_states, gate_up_weights, group_list=split_list, group_type=0)
@@ -39,10 +40,11 @@ def experts_computation(hidden_states, split_list, gate_up_weights, down_weights
     return npu_gmm_v2(act, down_weights, group_list=split_list, group_type=0)
 
 
-def dispatch_mlp_combine(hidden_states, top_k_index, top_k_weights, weights, num_global_experts=None):
+def dispatch_mlp_combine(hidden_states, top_k_index, top_k_weights, weights, num_global_experts=None,
+                         fuse_activation=False):
     gate_up_weights, down_weights = weights
     num_experts = gate_up_weights.size(0) if num_global_experts is None else num_global_experts
     permuted, row_id_map, _, tokens_per_expert = moe_token_permute_with_aux(
         hidden_states, top_k_index, num_experts=num_experts)
-    out = experts_computation(permuted, tokens_per_expert, gate_up_weights, down_weights)
+    out = experts_computation(permuted, tokens_per_expert, gate_up_weights, down_weights, fuse_activation)
     return npu_moe_token_unpermute(out, row_id_map, top_k_weights)

@@ -57,7 +57,7 @@ def _gmm_swiglu_forward(x, weight, group_list, group_list_type, probs):
     nbytes = ctypes.c_size_t(0)
     _lib.check(lib.ms_gmm_workspace_size(gl.numel(), m, 0, ctypes.byref(nbytes)), "ms_gmm_workspace_size")
     ws = _lib.workspace(nbytes.value, dev)
-    with torch.cuda.device(dev), flop_counter.op("gmm_fwd", flop_counter.gmm_flops(m, k, 2 * ffn), "flop", dev):
+    with torch.cuda.device(dev), flop_counter.op("gmm_fwd_swiglu", flop_counter.gmm_flops(m, k, 2 * ffn), "flop", dev):
         _lib.check(lib.ms_gmm_swiglu(
             _lib.stream_ptr(dev), _lib.ptr(x), x.stride(0), x.stride(1), _lib.ptr(weight), weight.stride(0),
             weight.stride(1), weight.stride(2), _lib.ptr(fc1), 2 * ffn, _lib.ptr(act), ffn, _lib.ptr(p), p_code,
@@ -180,7 +180,7 @@ class GroupedMLPFunction(torch.autograd.Function):
                    "ms_gmm_swiglu_grad_workspace_size")
         ws = _lib.workspace(nbytes.value, dev)
         wt = w2c.transpose(1, 2)       # [E, hidden, ffn] view: element (k, n) of group g is w2[g, n, k]
-        with torch.cuda.device(dev), flop_counter.op("gmm_dx", flop_counter.gmm_flops(m, hidden, ffn), "flop", dev):
+        with torch.cuda.device(dev), flop_counter.op("gmm_dx_swiglu", flop_counter.gmm_flops(m, hidden, ffn), "flop", dev):
             _lib.check(lib.ms_gmm_swiglu_grad(
                 _lib.stream_ptr(dev), _lib.ptr(dy), dy.stride(0), dy.stride(1), _lib.ptr(w2c), wt.stride(0),
                 wt.stride(1), wt.stride(2), _lib.ptr(fc1), two_ffn, _lib.ptr(p),
