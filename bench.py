@@ -158,7 +158,8 @@ def measure_routing_map_mode(cfg, device, x, idx, p, iters=20, warmup=5):
     t_ufb = timed(unpermute_fb)
     move = (T + rows) * H * elem       # rows read once + rows written once, either direction
     return {
-        "note": "routing-map (mask) form on the same routing; every call re-sorts the [T, E] mask on the device",
+        "note": "routing-map (mask) form on the same routing; event-timed loops of single ops, host launch "
+                "overhead included",
         "rows": rows,
         "permute_fwd": {"avg_ms": round(t_pf, 5), "gbs": round(move / t_pf / 1e6, 1)},
         "permute_fwd_bwd": {"avg_ms": round(t_pfb, 5), "gbs": round(2 * move / t_pfb / 1e6, 1)},

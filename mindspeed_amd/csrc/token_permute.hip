@@ -694,6 +694,125 @@ __global__ __launch_bounds__(256) void routing_map_probs_grad_kernel(const int32
     grad_probs[i] = static_cast<unsigned>(r) < static_cast<unsigned>(num_rows) ? grad_permuted_probs[r] : S(0);
 }
 
+// Mask mode, rows laid out and moved in one launch (no drop-and-pad, experts a power of two up to 16, so that
+// a 16-byte vector of the map holds whole tokens and byte position b of a vector always belongs to expert
+// b % E).  Every scatter workgroup counts, per expert column, the set entries of the tokens in front of its
+// own and of all tokens (byte-wise over the map, read from L2), turns that into the next free row of every
+// expert as seen from its first token, walks its own few tokens in order, and copies their rows.  Same
+// outputs as the sort-based path.
+__global__ __launch_bounds__(256) void routing_map_fused_kernel(
+    const v16 *__restrict__ tokens, v16 *__restrict__ permuted, const unsigned char *__restrict__ map, int num_tokens,
+    int E, int num_rows, int32_t *__restrict__ row_id_map, int32_t *__restrict__ sorted_flat,
+    int64_t *__restrict__ tokens_per_expert, int vecs_per_row, int lanes) {
+    extern __shared__ int lds[];     // before[16], total[16], base[16], rows[rows_per_block][E]
+    int *before = lds, *total = lds + 16, *base = lds + 32, *rows = lds + 48;
+    const int tid = threadIdx.x;
+    const int rows_per_block = 256 / lanes;
+    const int t0 = blockIdx.x * rows_per_block;
+    const int t1 = min(t0 + rows_per_block, num_tokens);
+    const int64_t n = static_cast<int64_t>(num_tokens) * E;
+    const int64_t split = static_cast<int64_t>(t0) * E;          // flat entries in front of this workgroup
+    if (tid < 32) lds[tid] = 0;
+    __syncthreads();
+    // counters per byte position of a vector (position b <-> expert b % E); folded per expert afterwards
+    int cb[16], ct[16];
+#pragma unroll
+    for (int b = 0; b < 16; ++b) cb[b] = ct[b] = 0;
+    const int64_t nvec = n / 16;
+    const v16 *mv = reinterpret_cast<const v16 *>(map);
+    for (int64_t v = tid; v < nvec; v += 256) {
+        const v16 w = mv[v];
+        const int64_t first = v * 16;
+        const bool all_before = first + 16 <= split;
+        const bool none_before = first >= split;
+#pragma unroll
+        for (int b = 0; b < 16; ++b) {
+            const int bit = ((w[b >> 2] >> (8 * (b & 3))) & 0xffu) != 0u ? 1 : 0;
+            ct[b] += bit;
+            cb[b] += (all_before || (!none_before && first + b < split)) ? bit : 0;
+        }
+    }
+    // entries past the last whole vector (n is not a multiple of 16 only for small maps)
+    for (int64_t i = nvec * 16 + tid; i < n; i += 256) {
+        const int bit = map[i] != 0 ? 1 : 0;
+        const int e = static_cast<int>(i % E);
+        atomicAdd(&total[e], bit);
+        if (i < split) atomicAdd(&before[e], bit);
+    }
+    // fold byte positions into experts, then lanes, then wavefronts
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        if (e >= E) break;
+        int sb = 0, st = 0;
+#pragma unroll
+        for (int b = 0; b < 16; ++b)
+            if ((b & (E - 1)) == e) { sb += cb[b]; st += ct[b]; }   // E is a power of two
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) {
+            sb += __shfl_down(sb, d, 64);
+            st += __shfl_down(st, d, 64);
+        }
+        if ((tid & 63) == 0) {
+            atomicAdd(&before[e], sb);
+            atomicAdd(&total[e], st);
+        }
+    }
+    __syncthreads();
+    if (tid < E) {
+        int first = 0;
+        for (int e = 0; e < tid; ++e) first += total[e];
+        base[tid] = first + before[tid];
+        if (blockIdx.x == 0 && tokens_per_expert != nullptr) tokens_per_expert[tid] = total[tid];
+    }
+    if (blockIdx.x == 0) {   // rows that nothing maps to (only if the caller's row count exceeds the set entries)
+        int nnz = 0;
+        for (int e = 0; e < E; ++e) nnz += total[e];
+        for (int r = nnz + tid; r < num_rows; r += 256) sorted_flat[r] = -1;
+    }
+    __syncthreads();
+    // own tokens, in order, one thread per expert column
+    if (tid < E) {
+        int next = base[tid];
+        for (int t = t0; t < t1; ++t) {
+            const int64_t i = static_cast<int64_t>(t) * E + tid;
+            int row = 0x7fffffff;
+            if (map[i] != 0) {
+                if (next < num_rows) {
+                    row = next;
+                    sorted_flat[row] = static_cast<int32_t>(i);
+                }
+                ++next;
+            }
+            row_id_map[i] = row;
+            rows[(t - t0) * E + tid] = row;
+        }
+    }
+    __syncthreads();
+    if (tokens == nullptr) return;
+    const int local_row = tid / lanes;
+    const int lane = tid % lanes;
+    const int t = t0 + local_row;
+    if (t >= num_tokens) return;
+    const v16 *src = tokens + static_cast<int64_t>(t) * vecs_per_row;
+    int d[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) d[j] = j < E ? rows[local_row * E + j] : 0x7fffffff;
+    for (int c0 = lane; c0 < vecs_per_row; c0 += 4 * lanes) {
+        v16 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            if (static_cast<unsigned>(d[j]) >= static_cast<unsigned>(num_rows)) continue;
+            v16 *dst = permuted + static_cast<int64_t>(d[j]) * vecs_per_row;
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (c0 + u * lanes < vecs_per_row) dst[c0 + u * lanes] = v[u];
+        }
+    }
+}
+
 // ---- host helpers -------------------------------------------------------------------
 struct SortPlan {
     int n, nbins, nbits, seg, nseg;
@@ -1019,6 +1138,23 @@ extern "C" int ms_moe_routing_map_permute(ms_stream_t stream_, const void *token
     if (T == 0) return MS_OK;
     MS_REQUIRE(routing_map && row_id_map && sorted_flat, MS_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", fn);
     MS_REQUIRE(tokens == nullptr || permuted != nullptr || num_rows == 0, MS_ERR_INVALID_ARGUMENT, "%s: permuted is NULL", fn);
+    // one launch when whole tokens fit a 16-byte vector of the map and rows move as 16-byte vectors
+    const int64_t row_bytes_f = H * dtype_size(dtype);
+    const bool pow2 = (E & (E - 1)) == 0 && E <= 16;
+    if (!drop_and_pad && pow2 && aligned16(routing_map) &&
+        (tokens == nullptr || (row_bytes_f % 16 == 0 && aligned16(tokens) && aligned16(permuted)))) {
+        const int64_t vecs = tokens != nullptr ? row_bytes_f / 16 : 1;
+        const RowLayout rl = tokens != nullptr ? row_layout(vecs) : RowLayout{1, 256};
+        const int64_t blocks = ceil_div(T, rl.rows_per_block);
+        const size_t lds = (48 + static_cast<size_t>(rl.rows_per_block) * E) * sizeof(int);
+        hipLaunchKernelGGL(routing_map_fused_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), lds, stream,
+                           static_cast<const v16 *>(tokens), static_cast<v16 *>(permuted),
+                           static_cast<const unsigned char *>(routing_map), static_cast<int>(T), static_cast<int>(E),
+                           static_cast<int>(num_rows), row_id_map, sorted_flat, tokens_per_expert, static_cast<int>(vecs),
+                           rl.lanes);
+        MS_CHECK_LAUNCH("routing_map_fused_kernel");
+        return MS_OK;
+    }
     const RoutingPlan r = make_routing_plan(T, E, drop_and_pad);
     MS_REQUIRE(workspace != nullptr && workspace_bytes >= r.total, MS_ERR_WORKSPACE_TOO_SMALL, "%s: workspace %zu < %zu bytes",
                fn, workspace_bytes, r.total);

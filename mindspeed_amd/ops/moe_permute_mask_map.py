@@ -94,6 +94,25 @@ def routing_map_row_maps(routing_map: torch.Tensor, num_rows: int, drop_and_pad:
     return permuted, row_id_map, sorted_flat, counts
 
 
+# The dispatcher hands the ``sorted_indices`` it got from ``permute`` back to ``unpermute`` together with the
+# same ``routing_map``.  The row map that ``permute`` computed from that mask travels along on the tensor, so
+# ``unpermute`` does not have to sort the mask again; it is only used when the mask is still the same tensor
+# in the same state (same storage, shape and version counter) and the row count and mode match.
+def _map_key(routing_map, num_rows, drop_and_pad):
+    return (routing_map.data_ptr(), tuple(routing_map.shape), routing_map._version, int(num_rows), bool(drop_and_pad))
+
+
+def _remember_row_map(sorted_indices, routing_map, row_id_map, drop_and_pad):
+    sorted_indices._ms_row_map = (_map_key(routing_map, sorted_indices.numel(), drop_and_pad), row_id_map)
+
+
+def _recall_row_map(sorted_indices, routing_map, num_rows, drop_and_pad):
+    cached = getattr(sorted_indices, "_ms_row_map", None)
+    if cached is not None and cached[0] == _map_key(routing_map, num_rows, drop_and_pad):
+        return cached[1]
+    return None
+
+
 def _resolve_num_rows(routing_map, num_out_tokens, drop_and_pad):
     if drop_and_pad:
         if num_out_tokens is None:
@@ -145,6 +164,7 @@ class MoePermuteMaskMap(torch.autograd.Function):
         ctx.num_rows = num_rows
         ctx.probs_dtype = probs.dtype if probs is not None else None
         ctx.mark_non_differentiable(sorted_indices)
+        _remember_row_map(sorted_indices, routing_map, row_id_map, drop_and_pad)
         return permuted, permuted_probs, sorted_indices
 
     @staticmethod
@@ -203,7 +223,9 @@ class MoeUnpermuteMaskMap(torch.autograd.Function):
         permuted_tokens = permuted_tokens.contiguous()
         num_experts = routing_map.size(1)
         num_rows, hidden = permuted_tokens.shape
-        _, row_id_map, _, _ = routing_map_row_maps(routing_map, num_rows, drop_and_pad)
+        row_id_map = _recall_row_map(sorted_indices, routing_map, num_rows, drop_and_pad)
+        if row_id_map is None:
+            _, row_id_map, _, _ = routing_map_row_maps(routing_map, num_rows, drop_and_pad)
         dev = permuted_tokens.device
         if probs is not None:
             _lib.require_device(probs, "probs")
