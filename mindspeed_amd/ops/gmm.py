@@ -204,6 +204,11 @@ class _beside:
             self.ctx.__exit__(*exc)
         return False
 
+    def again(self):
+        """A further ``with`` block on the side stream, ordered after what the caller's stream holds now (and,
+        being the same stream, after the earlier block)."""
+        return self
+
     def join(self):
         if self.active:
             self.main.wait_stream(self.side)

@@ -131,24 +131,60 @@ def _swiglu_from_fc1(fc1, p):
     return act
 
 
-class GroupedMLPFunction(torch.autograd.Function):
-    """The whole expert MLP of ``GmmExpertsImpl.forward`` (experts.py:113-160) as one autograd node, so that the
-    SwiGLU backward can ride on the epilogue of the second matmul's dX product:
+def _swiglu_grad_from_fc1(dact, fc1, p):
+    lib = _lib.load()
+    rows, two_ffn = fc1.shape
+    ffn = two_ffn // 2
+    dev = fc1.device
+    d_fc1 = torch.empty_like(fc1)
+    gp = torch.empty_like(p) if p is not None else None
+    with torch.cuda.device(dev), flop_counter.op(
+            "swiglu_grad", flop_counter.swiglu_bytes(rows, ffn, fc1.element_size(), True), "byte", dev):
+        _lib.check(lib.ms_swiglu_grad(_lib.stream_ptr(dev), _lib.ptr(dact), _lib.ptr(fc1), _lib.ptr(p),
+                                      _lib.dtype_code(p.dtype, "probs") if p is not None else 0, rows, ffn,
+                                      _lib.dtype_code(fc1.dtype, "x"), _lib.ptr(d_fc1), _lib.ptr(gp)), "ms_swiglu_grad")
+    return d_fc1, gp
 
-    forward   ``act = gmm_swiglu(x, w1)``; ``out = gmm(act, w2)``
-    backward  ``d_fc1, d_probs = [dy @ w2^T fused with SwiGLU backward on the saved fc1]``;
+
+class GroupedMLPFunction(torch.autograd.Function):
+    """The whole expert MLP of ``GmmExpertsImpl.forward`` (experts.py:113-160) as one autograd node:
+
+    forward   ``fc1 = gmm(x, w1)``; ``act = silu(gate) * up * probs``; ``out = gmm(act, w2)``
+    backward  ``dact = dy @ w2^T``; ``d_fc1, d_probs = SwiGLU backward on the saved fc1``;
               ``dW2 = act^T dy``; ``dx = d_fc1 @ w1^T``; ``dW1 = x^T d_fc1``
+
+    One node instead of three keeps a second stream busy from start to end of the backward pass: dW2 runs
+    beside dX2 and the SwiGLU backward, dW1 beside dX1, with one join at the very end (measured on the
+    Mixtral shape this is no faster than three nodes that each overlap their own dW: the step is limited by
+    board power, not by idle units).
+    ``fused_kernels``: the activation comes out of the first matmul's epilogue and its backward rides on the
+    epilogue of the dX2 product (16-bit, vector-access layout only); otherwise one kernel per op, any dtype.
     ``recompute_activation``: ``act`` is not kept; backward rebuilds it from ``fc1`` for dW2.
     """
 
     @staticmethod
-    def forward(ctx, x, w1, w2, group_list, group_list_type, probs, recompute_activation):
-        fc1, act, gl, p = _gmm_swiglu_forward(x, w1, group_list, group_list_type, probs)
+    def forward(ctx, x, w1, w2, group_list, group_list_type, probs, recompute_activation, fused_kernels):
+        if fused_kernels:
+            fc1, act, gl, p = _gmm_swiglu_forward(x, w1, group_list, group_list_type, probs)
+        else:
+            _lib.require_device(x, "x")
+            gl = _group_list_tensor(group_list, x.device)
+            fc1 = gmm_raw(x, w1, gl, 0, group_list_type)
+            p = None
+            if probs is not None:
+                _lib.require_device(probs, "probs")
+                p = probs.contiguous().view(-1)
+                if p.numel() != fc1.size(0):
+                    raise RuntimeError(f"probs has {p.numel()} entries, expected {fc1.size(0)}")
+            if fc1.size(1) % 2 != 0:
+                raise RuntimeError(f"the first matmul must produce an even number of columns, got {fc1.size(1)}")
+            act = _swiglu_from_fc1(fc1, p)
         if w2.dim() != 3 or w2.size(0) != w1.size(0) or w2.size(1) != act.size(1) or w2.dtype != x.dtype:
             raise ValueError(f"w2 {tuple(w2.shape)} {w2.dtype} does not match the activation {tuple(act.shape)} {act.dtype}")
         out = gmm_raw(act, w2, gl, 0, group_list_type)
         ctx.save_for_backward(x, w1, w2, gl, fc1, p, None if recompute_activation else act)
         ctx.group_list_type = group_list_type
+        ctx.fused_kernels = fused_kernels
         ctx.probs_shape = None if probs is None else probs.shape
         return out
 
@@ -159,47 +195,52 @@ class GroupedMLPFunction(torch.autograd.Function):
         dev = grad_out.device
         glt = ctx.group_list_type
         dy = grad_out.contiguous()
-        w2c = w2.contiguous()
         m, two_ffn = fc1.shape
         ffn = two_ffn // 2
         hidden = dy.size(1)
         num_groups = gl.numel()
         if act is None:
             act = _swiglu_from_fc1(fc1, p)
+        # everything the side stream writes is allocated here, on the caller's stream
         dw1 = torch.empty(w1.shape, dtype=w1.dtype, device=dev) if ctx.needs_input_grad[1] else None
         dw2 = torch.empty(w2.shape, dtype=w2.dtype, device=dev) if ctx.needs_input_grad[2] else None
-        # dW2 needs only act and dy: it runs beside the fused dX product
-        fork2 = _beside(dev)
-        with fork2:
+        side = _beside(dev)
+        with side:                                   # dW2 needs only act and dy
             if dw2 is not None:
                 gmm_raw(act.t(), dy, gl, 2, glt, out=dw2)
-        d_fc1 = torch.empty_like(fc1)
-        gp = torch.empty_like(p) if p is not None else None
-        nbytes = ctypes.c_size_t(0)
-        _lib.check(lib.ms_gmm_swiglu_grad_workspace_size(num_groups, m, ffn, ctypes.byref(nbytes)),
-                   "ms_gmm_swiglu_grad_workspace_size")
-        ws = _lib.workspace(nbytes.value, dev)
-        wt = w2c.transpose(1, 2)       # [E, hidden, ffn] view: element (k, n) of group g is w2[g, n, k]
-        with torch.cuda.device(dev), flop_counter.op("gmm_dx_swiglu", flop_counter.gmm_flops(m, hidden, ffn), "flop", dev):
-            _lib.check(lib.ms_gmm_swiglu_grad(
-                _lib.stream_ptr(dev), _lib.ptr(dy), dy.stride(0), dy.stride(1), _lib.ptr(w2c), wt.stride(0),
-                wt.stride(1), wt.stride(2), _lib.ptr(fc1), two_ffn, _lib.ptr(p),
-                _lib.dtype_code(p.dtype, "probs") if p is not None else 0, _lib.ptr(d_fc1), two_ffn, _lib.ptr(gp),
-                _lib.ptr(gl), glt, num_groups, m, hidden, ffn, _lib.dtype_code(dy.dtype, "grad"), _lib.ptr(ws),
-                ws.numel()), "ms_gmm_swiglu_grad")
-        fork2.join()
-        fork1 = _beside(dev)
-        with fork1:
+        if ctx.fused_kernels:
+            w2c = w2.contiguous()
+            d_fc1 = torch.empty_like(fc1)
+            gp = torch.empty_like(p) if p is not None else None
+            nbytes = ctypes.c_size_t(0)
+            _lib.check(lib.ms_gmm_swiglu_grad_workspace_size(num_groups, m, ffn, ctypes.byref(nbytes)),
+                       "ms_gmm_swiglu_grad_workspace_size")
+            ws = _lib.workspace(nbytes.value, dev)
+            wt = w2c.transpose(1, 2)       # [E, hidden, ffn] view: element (k, n) of group g is w2[g, n, k]
+            with torch.cuda.device(dev), flop_counter.op("gmm_dx_swiglu", flop_counter.gmm_flops(m, hidden, ffn),
+                                                         "flop", dev):
+                _lib.check(lib.ms_gmm_swiglu_grad(
+                    _lib.stream_ptr(dev), _lib.ptr(dy), dy.stride(0), dy.stride(1), _lib.ptr(w2c), wt.stride(0),
+                    wt.stride(1), wt.stride(2), _lib.ptr(fc1), two_ffn, _lib.ptr(p),
+                    _lib.dtype_code(p.dtype, "probs") if p is not None else 0, _lib.ptr(d_fc1), two_ffn, _lib.ptr(gp),
+                    _lib.ptr(gl), glt, num_groups, m, hidden, ffn, _lib.dtype_code(dy.dtype, "grad"), _lib.ptr(ws),
+                    ws.numel()), "ms_gmm_swiglu_grad")
+        else:
+            dact = gmm_raw(dy, w2.transpose(1, 2), gl, 0, glt)
+            d_fc1, gp = _swiglu_grad_from_fc1(dact, fc1, p)
+        with side.again():                           # dW1 needs d_fc1: the side stream picks up from here
             if dw1 is not None:
                 gmm_raw(x.t(), d_fc1, gl, 2, glt, out=dw1)
         dx = gmm_raw(d_fc1, w1.transpose(1, 2), gl, 0, glt) if ctx.needs_input_grad[0] else None
-        fork1.join()
+        side.join()
         gp_out = gp.view(ctx.probs_shape) if (gp is not None and ctx.needs_input_grad[5]) else None
-        return dx, dw1, dw2, None, None, gp_out, None
+        return dx, dw1, dw2, None, None, gp_out, None, None
 
 
-def grouped_mlp(x, w1, w2, group_list, probs=None, *, group_list_type: int = 1, recompute_activation: bool = False):
-    """``gmm(silu(gate) * up * probs, w2)`` with ``gate | up = gmm(x, w1)``: the expert MLP with both SwiGLU passes
-    fused into the neighbouring grouped matmuls.  ``w1 [E, K, 2*ffn]``, ``w2 [E, ffn, K']``; same layout conditions
-    as :func:`gmm_swiglu`."""
-    return GroupedMLPFunction.apply(x, w1, w2, group_list, group_list_type, probs, recompute_activation)
+def grouped_mlp(x, w1, w2, group_list, probs=None, *, group_list_type: int = 1, recompute_activation: bool = False,
+                fused_kernels: bool = True):
+    """``gmm(silu(gate) * up * probs, w2)`` with ``gate | up = gmm(x, w1)``: the expert MLP as one autograd node.
+    ``w1 [E, K, 2*ffn]``, ``w2 [E, ffn, K']``.  ``fused_kernels`` (default) fuses both SwiGLU passes into the
+    neighbouring grouped matmuls and needs the layout conditions of :func:`gmm_swiglu`; without it every op is
+    its own kernel, for any dtype and layout the grouped matmul takes."""
+    return GroupedMLPFunction.apply(x, w1, w2, group_list, group_list_type, probs, recompute_activation, fused_kernels)

@@ -115,8 +115,27 @@ MLP_CASES = [
 
 @pytest.mark.parametrize("counts,K,ffn,dtype,pdt,extra", MLP_CASES)
 @pytest.mark.parametrize("recompute", [False, True])
-def test_grouped_mlp_forward_backward(counts, K, ffn, dtype, pdt, extra, recompute, device):
-    say("grouped_mlp case", counts, K, ffn, dtype, pdt, extra, recompute)
+@pytest.mark.parametrize("fused_kernels", [True, False])
+def test_grouped_mlp_forward_backward(counts, K, ffn, dtype, pdt, extra, recompute, fused_kernels, device):
+    _grouped_mlp_case(counts, K, ffn, dtype, pdt, extra, recompute, fused_kernels, device)
+
+
+# layouts and dtypes only the one-kernel-per-op node takes: fp32, and sizes that rule out 16-byte accesses
+UNFUSED_ONLY_CASES = [
+    ([5, 0, 7, 3], 64, 96, torch.float32, torch.float32, 0),
+    ([33, 20, 0, 11], 36, 50, torch.bfloat16, torch.float32, 3),
+    ([17, 40], 30, 27, torch.float16, None, 0),
+]
+
+
+@pytest.mark.parametrize("counts,K,ffn,dtype,pdt,extra", UNFUSED_ONLY_CASES)
+def test_grouped_mlp_separate_kernels_any_layout(counts, K, ffn, dtype, pdt, extra, device):
+    _grouped_mlp_case(counts, K, ffn, dtype, pdt, extra, False, False, device)
+
+
+def _grouped_mlp_case(counts, K, ffn, dtype, pdt, extra, recompute, fused_kernels, device):
+    say("grouped_mlp case", counts, K, ffn, dtype, pdt, extra, recompute, fused_kernels)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
     E, M = len(counts), sum(counts) + extra
     gen = torch.Generator().manual_seed(M + ffn + 1)
     x = torch.randn(M, K, generator=gen).to(dtype)
@@ -139,23 +158,26 @@ def test_grouped_mlp_forward_backward(counts, K, ffn, dtype, pdt, extra, recompu
     out_sep.backward(gy.to(device))
 
     xf, w1f, w2f, pf = leaves()
-    out = ops.grouped_mlp(xf, w1f, w2f, gl.to(device), pf, recompute_activation=recompute)
+    out = ops.grouped_mlp(xf, w1f, w2f, gl.to(device), pf, recompute_activation=recompute,
+                          fused_kernels=fused_kernels)
     out.backward(gy.to(device))
     torch.cuda.synchronize()
     assert torch.equal(out, out_sep)
     assert torch.equal(xf.grad, xs.grad)                   # d_fc1 is bit-identical, so everything behind it is
     assert torch.equal(w1f.grad, w1s.grad) and torch.equal(w2f.grad, w2s.grad)
-    if probs is not None:
+    if probs is not None and fused_kernels:
         # same terms, summed per 64 columns and then over the row instead of in one pass
         assert rel_l2(pf.grad, ps.grad) <= (1e-5 if pdt == torch.float32 else 1e-2)
+    elif probs is not None:
+        assert torch.equal(pf.grad, ps.grad)               # the very same kernel
 
     x64, w164, w264 = (t.double().requires_grad_(True) for t in (x, w1, w2))
     p64 = None if probs is None else probs.double().requires_grad_(True)
     fc1_o = O.gmm(x64, w164, gl, group_type=0, group_list_type=1)
     out_o = O.gmm(O.swiglu(fc1_o, p64), w264, gl, group_type=0, group_list_type=1)
     out_o.backward(gy.double())
-    assert rel_l2(out, out_o) <= 1e-2
-    assert rel_l2(xf.grad, x64.grad) <= 1e-2
-    assert rel_l2(w1f.grad, w164.grad) <= 1e-2 and rel_l2(w2f.grad, w264.grad) <= 1e-2
+    assert rel_l2(out, out_o) <= tol
+    assert rel_l2(xf.grad, x64.grad) <= tol
+    assert rel_l2(w1f.grad, w164.grad) <= tol and rel_l2(w2f.grad, w264.grad) <= tol
     if probs is not None:
-        assert rel_l2(pf.grad, p64.grad) <= 1e-2
+        assert rel_l2(pf.grad, p64.grad) <= tol
