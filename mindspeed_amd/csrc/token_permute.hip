@@ -85,7 +85,8 @@ __device__ __forceinline__ void hist_keys(int *row, const int (&keys)[kKeysPerLa
 // the next output row of `key` for this wavefront's segment.  The lowest lane of every key fetches
 // and advances that counter with one returning LDS add and hands the old value to the key's lanes.
 __device__ __forceinline__ void scatter_keys(int *row, const int (&keys)[kKeysPerLane], int begin, int count,
-                                             int nbits, int num_out, int32_t *row_id_map, int32_t *sorted_indices) {
+                                             int nbits, int num_out, int32_t *row_id_map, int32_t *sorted_indices,
+                                             int *echo = nullptr, int echo_begin = 0) {
     const int lane = threadIdx.x & 63;
     const unsigned long long lt = (1ull << lane) - 1ull;
 #pragma unroll
@@ -102,6 +103,7 @@ __device__ __forceinline__ void scatter_keys(int *row, const int (&keys)[kKeysPe
             const int rank = first + __popcll(m & lt);
             const int i = begin + u * 64 + lane;
             row_id_map[i] = rank;
+            if (echo != nullptr) echo[i - echo_begin] = rank;
             if (sorted_indices != nullptr && rank < num_out) sorted_indices[rank] = i;
         }
     }
@@ -136,7 +138,8 @@ __device__ __forceinline__ void hist_keys_few(int *row, const int (&keys)[kKeysP
 
 template <int NB>
 __device__ __forceinline__ void scatter_keys_few(int *row, const int (&keys)[kKeysPerLane], int begin, int count,
-                                                 int nbins, int num_out, int32_t *row_id_map, int32_t *sorted_indices) {
+                                                 int nbins, int num_out, int32_t *row_id_map, int32_t *sorted_indices,
+                                                 int *echo = nullptr, int echo_begin = 0) {
     const int lane = threadIdx.x & 63;
     int base[NB];
     const int mine = lane < nbins ? row[lane] : 0;
@@ -155,6 +158,7 @@ __device__ __forceinline__ void scatter_keys_few(int *row, const int (&keys)[kKe
         if (keys[u] >= 0) {
             const int i = begin + u * 64 + lane;
             row_id_map[i] = rank;
+            if (echo != nullptr) echo[i - echo_begin] = rank;
             if (sorted_indices != nullptr && rank < num_out) sorted_indices[rank] = i;
         }
     }
@@ -170,11 +174,16 @@ __device__ __forceinline__ void hist_chunk(int *row, const int (&keys)[kKeysPerL
     else if (nbins <= 16) hist_keys_few<16>(row, keys, count, nbins);
     else hist_keys(row, keys, count, nbits);
 }
+// `echo` (optional, LDS): the row of flat position i is also written to echo[i - echo_begin].
 __device__ __forceinline__ void scatter_chunk(int *row, const int (&keys)[kKeysPerLane], int begin, int count, int nbins,
-                                              int nbits, int num_out, int32_t *row_id_map, int32_t *sorted_indices) {
-    if (nbins <= 8) scatter_keys_few<8>(row, keys, begin, count, nbins, num_out, row_id_map, sorted_indices);
-    else if (nbins <= 16) scatter_keys_few<16>(row, keys, begin, count, nbins, num_out, row_id_map, sorted_indices);
-    else scatter_keys(row, keys, begin, count, nbits, num_out, row_id_map, sorted_indices);
+                                              int nbits, int num_out, int32_t *row_id_map, int32_t *sorted_indices,
+                                              int *echo = nullptr, int echo_begin = 0) {
+    if (nbins <= 8)
+        scatter_keys_few<8>(row, keys, begin, count, nbins, num_out, row_id_map, sorted_indices, echo, echo_begin);
+    else if (nbins <= 16)
+        scatter_keys_few<16>(row, keys, begin, count, nbins, num_out, row_id_map, sorted_indices, echo, echo_begin);
+    else
+        scatter_keys(row, keys, begin, count, nbits, num_out, row_id_map, sorted_indices, echo, echo_begin);
 }
 
 // Histogram of idx[begin, end) into one table row owned by this wavefront.
@@ -193,12 +202,12 @@ __device__ __forceinline__ void wave_histogram(int *row, const IdxT *idx, int be
 template <typename IdxT>
 __device__ __forceinline__ void wave_scatter(int *row, const IdxT *idx, int begin, int end,
                                              int nbins, int nbits, int num_out, int32_t *row_id_map,
-                                             int32_t *sorted_indices) {
+                                             int32_t *sorted_indices, int *echo = nullptr) {
     int keys[kKeysPerLane];
     for (int c = begin; c < end; c += kChunk) {
         const int ce = min(c + kChunk, end);
         load_keys(idx, c, ce, nbins, keys);
-        scatter_chunk(row, keys, c, ce - c, nbins, nbits, num_out, row_id_map, sorted_indices);
+        scatter_chunk(row, keys, c, ce - c, nbins, nbits, num_out, row_id_map, sorted_indices, echo, begin);
     }
 }
 
@@ -381,9 +390,9 @@ __global__ __launch_bounds__(256) void permute_rows_kernel(const VecT *__restric
 
 // out[t] = sum_j w[t,j] * rows[row_id_map[t*k+j]] ; w == nullptr -> unweighted.
 // VEC: elements per thread access (16 bytes worth, or 1 for the unaligned path).
-// Row ids and weights are read once per thread; per pair of output vectors all topk row loads are
-// independent and issued together; accumulation is fp32 in registers, one rounding.
-template <typename DT, int VEC>
+// Row ids and weights are read once per thread; per group of U output vectors the row loads of up to JB
+// slots are independent and issued together; accumulation is fp32 in registers, slot by slot, one rounding.
+template <typename DT, int VEC, int JB, int U>
 __global__ __launch_bounds__(256) void gather_combine_kernel(
     const typename DT::storage *__restrict__ rows, const int32_t *__restrict__ row_id_map,
     const typename DT::storage *__restrict__ probs, typename DT::storage *__restrict__ out,
@@ -394,25 +403,24 @@ __global__ __launch_bounds__(256) void gather_combine_kernel(
     const int t = blockIdx.x * (256 / lanes) + local_row;
     if (t >= num_tokens) return;
     const int vecs = hidden / VEC;
-    constexpr int U = 2;
     for (int c0 = lane; c0 < vecs; c0 += U * lanes) {
         float acc[U][VEC];
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int e = 0; e < VEC; ++e) acc[u][e] = 0.f;
-        for (int j0 = 0; j0 < topk; j0 += kSlotBatch) {
-            int d[kSlotBatch];
-            float w[kSlotBatch];
+        for (int j0 = 0; j0 < topk; j0 += JB) {
+            int d[JB];
+            float w[JB];
 #pragma unroll
-            for (int j = 0; j < kSlotBatch; ++j) {
+            for (int j = 0; j < JB; ++j) {
                 const int64_t flat = static_cast<int64_t>(t) * topk + j0 + j;
                 d[j] = j0 + j < topk ? row_id_map[flat] : num_rows;
                 w[j] = (probs != nullptr && j0 + j < topk) ? DT::to_float(probs[flat]) : 1.f;
             }
-            S tmp[kSlotBatch][U][VEC];
+            S tmp[JB][U][VEC];
 #pragma unroll
-            for (int j = 0; j < kSlotBatch; ++j) {
+            for (int j = 0; j < JB; ++j) {
                 if (static_cast<unsigned>(d[j]) >= static_cast<unsigned>(num_rows)) continue;
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -428,7 +436,7 @@ __global__ __launch_bounds__(256) void gather_combine_kernel(
                 }
             }
 #pragma unroll
-            for (int j = 0; j < kSlotBatch; ++j) {
+            for (int j = 0; j < JB; ++j) {
                 if (static_cast<unsigned>(d[j]) >= static_cast<unsigned>(num_rows)) continue;
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -456,69 +464,97 @@ __global__ __launch_bounds__(256) void gather_combine_kernel(
     }
 }
 
-// One block per token: grad_permuted[row] = w * dY[t]; grad_probs[t,j] = <dY[t], permuted[row]>.
-template <typename DT, int VEC>
+// grad_permuted[row] = w * dY[t]; grad_probs[t,j] = <dY[t], permuted[row]> for row = row_id_map[t*k+j].
+// `lanes` threads (a power of two, one wavefront at most) share a token, so the dot products are folded with
+// lane shuffles and the kernel has no barrier.  Per chunk of U vectors a thread reads dY once and has the
+// loads of up to JB slots' rows in flight together.
+template <typename DT, int VEC, int JB, int U>
 __global__ __launch_bounds__(256) void unpermute_grad_kernel(
     const typename DT::storage *__restrict__ permuted, const typename DT::storage *__restrict__ grad_out,
     const int32_t *__restrict__ row_id_map, const typename DT::storage *__restrict__ probs,
     typename DT::storage *__restrict__ grad_permuted, typename DT::storage *__restrict__ grad_probs,
-    int topk, int hidden, int num_rows) {
+    int num_tokens, int topk, int hidden, int num_rows, int lanes) {
     using S = typename DT::storage;
-    __shared__ float partial[4];
-    const int t = blockIdx.x;
+    const int local_row = threadIdx.x / lanes;
+    const int lane = threadIdx.x % lanes;
+    const int t = blockIdx.x * (256 / lanes) + local_row;
+    if (t >= num_tokens) return;
     const int vecs = hidden / VEC;
     const S *gy = grad_out + static_cast<int64_t>(t) * hidden;
-    for (int j = 0; j < topk; ++j) {
-        const int64_t flat = static_cast<int64_t>(t) * topk + j;
-        const int d = row_id_map[flat];
-        const bool kept = static_cast<unsigned>(d) < static_cast<unsigned>(num_rows);   // negative ids count as dropped
-        const float w = probs != nullptr ? DT::to_float(probs[flat]) : 1.f;
-        float dot = 0.f;
-        if (kept) {
-            for (int c = threadIdx.x; c < vecs; c += blockDim.x) {
-                S g[VEC], x[VEC], o[VEC];
+    const bool want_dot = grad_probs != nullptr;
+    for (int j0 = 0; j0 < topk; j0 += JB) {
+        int d[JB];
+        float w[JB], dot[JB];
+#pragma unroll
+        for (int j = 0; j < JB; ++j) {
+            const int64_t flat = static_cast<int64_t>(t) * topk + j0 + j;
+            d[j] = j0 + j < topk ? row_id_map[flat] : num_rows;          // ids outside [0, num_rows): dropped
+            w[j] = (probs != nullptr && j0 + j < topk) ? DT::to_float(probs[flat]) : 1.f;
+            dot[j] = 0.f;
+        }
+        for (int c0 = lane; c0 < vecs; c0 += U * lanes) {
+            S g[U][VEC], x[JB][U][VEC];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u * lanes;
+                if (c >= vecs) continue;
                 const S *gp = gy + static_cast<int64_t>(c) * VEC;
-                const int64_t off = static_cast<int64_t>(d) * hidden + static_cast<int64_t>(c) * VEC;
                 if constexpr (VEC * sizeof(S) == 16) {
-                    *reinterpret_cast<v16 *>(g) = *reinterpret_cast<const v16 *>(gp);
-                    if (grad_probs != nullptr)
-                        *reinterpret_cast<v16 *>(x) =
-                            MS_NT_LOAD(reinterpret_cast<const v16 *>(permuted + off));
+                    *reinterpret_cast<v16 *>(g[u]) = *reinterpret_cast<const v16 *>(gp);
                 } else {
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) g[e] = gp[e];
-                    if (grad_probs != nullptr) {
+                    for (int e = 0; e < VEC; ++e) g[u][e] = gp[e];
+                }
+            }
+            if (want_dot) {
 #pragma unroll
-                        for (int e = 0; e < VEC; ++e) x[e] = permuted[off + e];
+                for (int j = 0; j < JB; ++j) {
+                    if (static_cast<unsigned>(d[j]) >= static_cast<unsigned>(num_rows)) continue;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int c = c0 + u * lanes;
+                        if (c >= vecs) continue;
+                        const S *xp = permuted + static_cast<int64_t>(d[j]) * hidden + static_cast<int64_t>(c) * VEC;
+                        if constexpr (VEC * sizeof(S) == 16) {
+                            *reinterpret_cast<v16 *>(x[j][u]) = MS_NT_LOAD(reinterpret_cast<const v16 *>(xp));
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < VEC; ++e) x[j][u][e] = xp[e];
+                        }
                     }
                 }
+            }
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const float gf = DT::to_float(g[e]);
-                    o[e] = DT::from_float(w * gf);
-                    if (grad_probs != nullptr) dot = fmaf(gf, DT::to_float(x[e]), dot);
-                }
-                if constexpr (VEC * sizeof(S) == 16) {
-                    MS_NT_STORE(*reinterpret_cast<v16 *>(o),
-                                                reinterpret_cast<v16 *>(grad_permuted + off));
-                } else {
+            for (int j = 0; j < JB; ++j) {
+                if (static_cast<unsigned>(d[j]) >= static_cast<unsigned>(num_rows)) continue;
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) grad_permuted[off + e] = o[e];
+                for (int u = 0; u < U; ++u) {
+                    const int c = c0 + u * lanes;
+                    if (c >= vecs) continue;
+                    S o[VEC];
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        const float gf = DT::to_float(g[u][e]);
+                        o[e] = DT::from_float(w[j] * gf);
+                        if (want_dot) dot[j] = fmaf(gf, DT::to_float(x[j][u][e]), dot[j]);
+                    }
+                    S *op = grad_permuted + static_cast<int64_t>(d[j]) * hidden + static_cast<int64_t>(c) * VEC;
+                    if constexpr (VEC * sizeof(S) == 16) {
+                        MS_NT_STORE(*reinterpret_cast<v16 *>(o), reinterpret_cast<v16 *>(op));
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) op[e] = o[e];
+                    }
                 }
             }
         }
-        if (grad_probs != nullptr) {
+        if (want_dot) {
 #pragma unroll
-            for (int dlt = 32; dlt > 0; dlt >>= 1) dot += __shfl_down(dot, dlt, 64);
-            const int wave = threadIdx.x >> 6;
-            if ((threadIdx.x & 63) == 0) partial[wave] = dot;
-            __syncthreads();
-            if (threadIdx.x == 0) {
-                float s = 0.f;
-                for (int w2 = 0; w2 < (blockDim.x + 63) / 64; ++w2) s += partial[w2];
-                grad_probs[flat] = DT::from_float(s);
+            for (int j = 0; j < JB; ++j) {
+                float s = dot[j];
+                for (int dlt = lanes >> 1; dlt > 0; dlt >>= 1) s += __shfl_xor(s, dlt, 64);
+                if (lane == 0 && j0 + j < topk) grad_probs[static_cast<int64_t>(t) * topk + j0 + j] = DT::from_float(s);
             }
-            __syncthreads();
         }
     }
 }
@@ -534,95 +570,175 @@ __global__ void copy_tail_kernel(const unsigned char *src, unsigned char *dst, s
     if (i < end) dst[i] = src[i];
 }
 
-// ---- sort + row scatter in one launch (small inputs, few bins) ------------------------------------
-// The single-workgroup sort is latency, not work: ~12 us for 8192 keys, after which the row scatter still has to
-// be launched.  Here every scatter workgroup works out the rows of its own tokens itself: its four wavefronts
-// count, per bin, the keys in front of the workgroup's first flat position and the keys from there on (two
-// histograms over all keys, read from L2 after the first workgroup has touched them), a scan over the bins
-// turns that into each bin's next free row as seen from this workgroup, and wavefront 0 ranks the
-// workgroup's own positions with the same stable scatter the sort kernels use.  Counting is redundant across
-// workgroups (every one reads all keys) but cheap, and it overlaps with the row traffic of the workgroups
-// that are already copying.  The integer outputs are the same as the sort kernels' by construction.
-constexpr int kFusedMaxBins = 16;   // the per-bin ballot counting; measured slower than two launches with 1024 bins
+// ---- sort and row scatter in one launch ------------------------------------------------
+constexpr int kFusedMaxBins = 16;     // one private LDS counter column per thread and bin; more bins: two launches
+constexpr int kFusedMaxLocal = 4096;  // flat positions of one workgroup whose rows are handed over through LDS
 
-template <typename IdxT, typename VecT>
-__global__ __launch_bounds__(256) void permute_fused_kernel(
+// Key of a raw index, clamped to [0, last] like load_keys does.  The quick form looks at the low half of a
+// 64-bit index only and reports (`bad`) whether any high half was set; the caller then counts again exactly.
+template <bool EXACT>
+__device__ __forceinline__ int fused_key(int32_t raw, int last, unsigned &) {
+    return min(max(raw, 0), last);
+}
+template <bool EXACT>
+__device__ __forceinline__ int fused_key(int64_t raw, int last, unsigned &bad) {
+    if constexpr (EXACT) {
+        const long long v = raw < 0 ? 0 : raw;
+        return static_cast<int>(v > last ? last : v);
+    } else {
+        bad |= static_cast<unsigned>(static_cast<unsigned long long>(raw) >> 32);
+        return static_cast<int>(min(static_cast<unsigned>(raw), static_cast<unsigned>(last)));
+    }
+}
+
+constexpr int kFusedKeys = 8;         // keys per thread in flight at a time
+
+// One batch of raw indices: flat positions c + u * blockDim.x + tid.
+template <typename IdxT>
+__device__ __forceinline__ void fused_load(IdxT (&raw)[kFusedKeys], const IdxT *__restrict__ idx, int c, int n) {
+#pragma unroll
+    for (int u = 0; u < kFusedKeys; ++u)
+        raw[u] = idx[min(c + u * static_cast<int>(blockDim.x) + static_cast<int>(threadIdx.x), n - 1)];
+}
+
+// Add the batch to the counter table: table[bin][tid % 256] for positions in front of `split`,
+// table[NB + bin][tid % 256] for the others, with fire-and-forget LDS adds.
+template <typename IdxT, int NB, bool EXACT>
+__device__ __forceinline__ void fused_add(int *table, const IdxT (&raw)[kFusedKeys], int c, int n, int split, int last,
+                                          unsigned &bad) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < kFusedKeys; ++u) {
+        const int pos = c + u * static_cast<int>(blockDim.x) + tid;
+        const int key = fused_key<EXACT>(raw[u], last, bad);
+        // positions past the end read the last index again and add nothing: straight-line code, so the
+        // waits stay per load
+        __hip_atomic_fetch_add(table + ((pos < split ? 0 : NB) + key) * 256 + (tid & 255), pos < n ? 1 : 0,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+}
+
+// sums[r] = sum of the 256 columns of table row r, for the 2 NB rows; the first 256 threads do it,
+// 256 / (2 NB) threads per row with 2 NB columns each.
+template <int NB>
+__device__ __forceinline__ void fused_fold(const int *table, int *sums) {
+    const int tid = threadIdx.x;
+    if (tid >= 256) return;
+    constexpr int TPR = 256 / (2 * NB);
+    constexpr int CPT = 2 * NB;
+    const int r = tid / TPR, part = tid % TPR;
+    int acc = 0;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) acc += table[r * 256 + ((j + part) % CPT) * TPR + part];
+#pragma unroll
+    for (int d = TPR >> 1; d > 0; d >>= 1) acc += __shfl_xor(acc, d, 64);
+    if (part == 0) sums[r] = acc;
+}
+
+// Sort and row scatter in one launch, for at most kFusedMaxBins keys and inputs one workgroup can count
+// (n <= kSmallSortMax).  Every workgroup (256, 512 or 1024 threads) moves the rows of rows_per_block tokens.  To
+// place them it needs, per key, the number of flat positions in front of its own (-> rank of its first
+// entry) and the total (-> first row of the key): it counts all n keys itself into 256 LDS counter columns,
+// folds the columns, and ranks its own positions with the same stable scatter the sort kernels use, which
+// also writes this workgroup's part of row_id_map / sorted_indices.  The counting is redundant across
+// workgroups but short (the keys come from L2) and needs no communication between workgroups; the first
+// vectors of the workgroup's source rows are requested before it starts, so the row reads are under way while
+// it runs.  The destination rows reach the copying threads through LDS.  The integer outputs are the same
+// as the sort kernels' by construction.
+template <typename IdxT, typename VecT, int NB>
+__global__ __launch_bounds__(1024) void permute_fused_kernel(
     const VecT *__restrict__ tokens, VecT *__restrict__ permuted, const IdxT *__restrict__ idx, int n, int nbins,
     int nbits, int num_out, int32_t *__restrict__ row_id_map, int32_t *__restrict__ sorted_indices,
     int64_t *__restrict__ tokens_per_expert, int tpe_n, int num_tokens, int topk, int vecs_per_row, int lanes) {
-    extern __shared__ int lds[];               // before[4][nbins], after[4][nbins], base[nbins], 16 ints scratch
-    int *before = lds;
-    int *after = lds + 4 * nbins;
-    int *base = lds + 8 * nbins;
-    int *scratch = base + nbins;
+    extern __shared__ int lds[];               // table[2 * NB][256], sums[2 * NB], base[NB], dest[rows_per_block * topk]
+    int *table = lds;
+    int *sums = lds + 2 * NB * 256;
+    int *base = sums + 2 * NB;
+    int *dest = base + NB;
     const int tid = threadIdx.x;
-    const int wave = tid >> 6;
-    const int rows_per_block = 256 / lanes;
+    const int nthreads = blockDim.x;
+    const int rows_per_block = nthreads / lanes;
     const int t0 = blockIdx.x * rows_per_block;
     const int t1 = min(t0 + rows_per_block, num_tokens);
     const int p0 = t0 * topk, p1 = t1 * topk;  // this workgroup's flat positions
-    for (int i = tid; i < 8 * nbins; i += 256) lds[i] = 0;
-    __syncthreads();
-    int seg = (n + 3) / 4;
-    seg = (seg + 63) & ~63;
-    const int b = min(wave * seg, n);
-    const int e = min(b + seg, n);
-    const int mid = min(max(p0, b), e);
-    wave_histogram(before + wave * nbins, idx, b, mid, nbins, nbits);
-    wave_histogram(after + wave * nbins, idx, mid, e, nbins, nbits);
-    __syncthreads();
-    // bins in passes of 256 (one per thread), the running row count carried from pass to pass
-    int carry = 0;
-    for (int e0 = 0; e0 < nbins; e0 += 256) {
-        const int bin = e0 + tid;
-        int bef = 0, tot = 0;
-        if (bin < nbins) {
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                bef += before[w * nbins + bin];
-                tot += after[w * nbins + bin];
-            }
-            tot += bef;
-        }
-        const int first = carry + block_exclusive_scan(tot, scratch);   // first row of this bin
-        if (bin < nbins) {
-            base[bin] = first + bef;
-            if (blockIdx.x == 0 && tokens_per_expert != nullptr && bin < tpe_n) tokens_per_expert[bin] = tot;
-        }
-        if (tid == 255) scratch[15] = first + tot;
-        __syncthreads();
-        carry = scratch[15];
-        __syncthreads();
-    }
-    if (wave == 0) wave_scatter(base, idx, p0, p1, nbins, nbits, num_out, row_id_map, sorted_indices);
-    // Workgroup-scope release / acquire (part of __syncthreads) is all the other wavefronts need to see the
-    // row ids: they run on the same compute unit.  A device-scope fence here would write the L2 back, rows
-    // of other workgroups included, once per workgroup.
-    __syncthreads();
-
     const int local_row = tid / lanes;
     const int lane = tid % lanes;
     const int t = t0 + local_row;
-    if (t >= num_tokens) return;
-    const VecT *src = tokens + static_cast<int64_t>(t) * vecs_per_row;
-    for (int j0 = 0; j0 < topk; j0 += kSlotBatch) {
-        int d[kSlotBatch];
+    const bool mover = t < num_tokens;
+    const VecT *src = tokens + static_cast<int64_t>(mover ? t : 0) * vecs_per_row;
+
+    if (tid < 256) {
 #pragma unroll
-        for (int j = 0; j < kSlotBatch; ++j)
-            d[j] = j0 + j < topk ? row_id_map[static_cast<int64_t>(t) * topk + j0 + j] : num_out;
-        for (int c0 = lane; c0 < vecs_per_row; c0 += 4 * lanes) {
-            VecT v[4];
+        for (int r = 0; r < 2 * NB; ++r) table[r * 256 + tid] = 0;
+    }
+    IdxT raw[kFusedKeys];
+    fused_load(raw, idx, 0, n);
+    // the workgroup's own indices, for the ranking below (first wavefront, up to 64 of them)
+    const bool few_own = p1 - p0 <= 64;
+    IdxT own = 0;
+    if (tid < 64) own = idx[min(p0 + tid, n - 1)];
+    VecT v[8];   // the first vectors of this thread's row; unconditional loads from clamped positions, so that
+                 // the waits for the indices above can leave these in flight
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+    for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+    __syncthreads();
+    unsigned bad = 0;
+    fused_add<IdxT, NB, false>(table, raw, 0, n, p0, nbins - 1, bad);
+    for (int c = kFusedKeys * nthreads; c < n; c += kFusedKeys * nthreads) {
+        fused_load(raw, idx, c, n);
+        fused_add<IdxT, NB, false>(table, raw, c, n, p0, nbins - 1, bad);
+    }
+    if (__syncthreads_or(bad != 0u)) {          // some index does not fit 32 bits: count again with the full clamp
+        if (tid < 256) {
+#pragma unroll
+            for (int r = 0; r < 2 * NB; ++r) table[r * 256 + tid] = 0;
+        }
+        __syncthreads();
+        for (int c = 0; c < n; c += kFusedKeys * nthreads) {
+            fused_load(raw, idx, c, n);
+            fused_add<IdxT, NB, true>(table, raw, c, n, p0, nbins - 1, bad);
+        }
+        __syncthreads();
+    }
+    fused_fold<NB>(table, sums);
+    __syncthreads();
+    if (tid < nbins) {
+        int first = 0;
+        for (int e = 0; e < tid; ++e) first += sums[e] + sums[NB + e];
+        base[tid] = first + sums[tid];
+        if (blockIdx.x == 0 && tokens_per_expert != nullptr && tid < tpe_n)
+            tokens_per_expert[tid] = sums[tid] + sums[NB + tid];
+    }
+    __syncthreads();
+    if (tid < 64) {
+        if (few_own) {
+            int keys[kKeysPerLane];
+#pragma unroll
+            for (int u = 1; u < kKeysPerLane; ++u) keys[u] = -1;
+            unsigned unused = 0;
+            keys[0] = p0 + tid < p1 ? fused_key<true>(own, nbins - 1, unused) : -1;
+            scatter_keys_few<NB>(base, keys, p0, p1 - p0, nbins, num_out, row_id_map, sorted_indices, dest, p0);
+        } else {
+            wave_scatter(base, idx, p0, p1, nbins, nbits, num_out, row_id_map, sorted_indices, dest);
+        }
+    }
+    __syncthreads();
+
+    if (!mover) return;
+    const int *d = dest + local_row * topk;
+    for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
+        if (c0 != lane) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
                 if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
+        }
+        for (int j = 0; j < topk; ++j) {
+            const int row = d[j];
+            if (static_cast<unsigned>(row) >= static_cast<unsigned>(num_out)) continue;   // dropped
+            VecT *dst = permuted + static_cast<int64_t>(row) * vecs_per_row;
 #pragma unroll
-            for (int j = 0; j < kSlotBatch; ++j) {
-                if (static_cast<unsigned>(d[j]) >= static_cast<unsigned>(num_out)) continue;   // dropped (or corrupt) id
-                VecT *dst = permuted + static_cast<int64_t>(d[j]) * vecs_per_row;
-#pragma unroll
-                for (int u = 0; u < 4; ++u)
-                    if (c0 + u * lanes < vecs_per_row) dst[c0 + u * lanes] = v[u];
-            }
+            for (int u = 0; u < 8; ++u)
+                if (c0 + u * lanes < vecs_per_row) dst[c0 + u * lanes] = v[u];
         }
     }
 }
@@ -696,118 +812,124 @@ __global__ __launch_bounds__(256) void routing_map_probs_grad_kernel(const int32
 
 // Mask mode, rows laid out and moved in one launch (no drop-and-pad, experts a power of two up to 16, so that
 // a 16-byte vector of the map holds whole tokens and byte position b of a vector always belongs to expert
-// b % E).  Every scatter workgroup counts, per expert column, the set entries of the tokens in front of its
-// own and of all tokens (byte-wise over the map, read from L2), turns that into the next free row of every
-// expert as seen from its first token, walks its own few tokens in order, and copies their rows.  Same
-// outputs as the sort-based path.
-__global__ __launch_bounds__(256) void routing_map_fused_kernel(
+// b % E; maps up to kFusedMapMax entries).  Same scheme as permute_fused_kernel: every workgroup counts, per
+// expert column, the set entries of the tokens in front of its own and of the others into 256 LDS counter
+// columns (the map comes from L2), folds them into the next free row of every expert as seen from its first
+// token, ranks its own entries in order with wavefront ballots, and copies its tokens' rows, whose first
+// vectors were requested before the counting.  Same outputs as the sort-based path.
+constexpr int kFusedMapMax = 1 << 17;
+
+__device__ __forceinline__ void mask_vector_add(int *table, const v16 &w, int first, int live, int split, int E) {
+    const int col = threadIdx.x & 255;
+#pragma unroll
+    for (int b = 0; b < 16; ++b) {
+        const unsigned byte = (w[b >> 2] >> (8 * (b & 3))) & 0xffu;
+        const int row = (first + b < split ? 0 : 16) + (b & (E - 1));
+        __hip_atomic_fetch_add(table + row * 256 + col, static_cast<int>(min(byte, 1u)) & live, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+}
+
+__global__ __launch_bounds__(1024) void routing_map_fused_kernel(
     const v16 *__restrict__ tokens, v16 *__restrict__ permuted, const unsigned char *__restrict__ map, int num_tokens,
     int E, int num_rows, int32_t *__restrict__ row_id_map, int32_t *__restrict__ sorted_flat,
     int64_t *__restrict__ tokens_per_expert, int vecs_per_row, int lanes) {
-    extern __shared__ int lds[];     // before[16], total[16], base[16], rows[rows_per_block][E]
-    int *before = lds, *total = lds + 16, *base = lds + 32, *rows = lds + 48;
+    extern __shared__ int lds[];     // table[32][256], sums[32], base[16], rows[rows_per_block * E]
+    int *table = lds;
+    int *sums = lds + 32 * 256;
+    int *base = sums + 32;
+    int *rows = base + 16;
     const int tid = threadIdx.x;
-    const int rows_per_block = 256 / lanes;
+    const int nthreads = blockDim.x;
+    const int rows_per_block = nthreads / lanes;
     const int t0 = blockIdx.x * rows_per_block;
     const int t1 = min(t0 + rows_per_block, num_tokens);
-    const int64_t n = static_cast<int64_t>(num_tokens) * E;
-    const int64_t split = static_cast<int64_t>(t0) * E;          // flat entries in front of this workgroup
-    if (tid < 32) lds[tid] = 0;
-    __syncthreads();
-    // counters per byte position of a vector (position b <-> expert b % E); folded per expert afterwards
-    int cb[16], ct[16];
-#pragma unroll
-    for (int b = 0; b < 16; ++b) cb[b] = ct[b] = 0;
-    const int64_t nvec = n / 16;
-    const v16 *mv = reinterpret_cast<const v16 *>(map);
-    for (int64_t v = tid; v < nvec; v += 256) {
-        const v16 w = mv[v];
-        const int64_t first = v * 16;
-        const bool all_before = first + 16 <= split;
-        const bool none_before = first >= split;
-#pragma unroll
-        for (int b = 0; b < 16; ++b) {
-            const int bit = ((w[b >> 2] >> (8 * (b & 3))) & 0xffu) != 0u ? 1 : 0;
-            ct[b] += bit;
-            cb[b] += (all_before || (!none_before && first + b < split)) ? bit : 0;
-        }
-    }
-    // entries past the last whole vector (n is not a multiple of 16 only for small maps)
-    for (int64_t i = nvec * 16 + tid; i < n; i += 256) {
-        const int bit = map[i] != 0 ? 1 : 0;
-        const int e = static_cast<int>(i % E);
-        atomicAdd(&total[e], bit);
-        if (i < split) atomicAdd(&before[e], bit);
-    }
-    // fold byte positions into experts, then lanes, then wavefronts
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-        if (e >= E) break;
-        int sb = 0, st = 0;
-#pragma unroll
-        for (int b = 0; b < 16; ++b)
-            if ((b & (E - 1)) == e) { sb += cb[b]; st += ct[b]; }   // E is a power of two
-#pragma unroll
-        for (int d = 32; d > 0; d >>= 1) {
-            sb += __shfl_down(sb, d, 64);
-            st += __shfl_down(st, d, 64);
-        }
-        if ((tid & 63) == 0) {
-            atomicAdd(&before[e], sb);
-            atomicAdd(&total[e], st);
-        }
-    }
-    __syncthreads();
-    if (tid < E) {
-        int first = 0;
-        for (int e = 0; e < tid; ++e) first += total[e];
-        base[tid] = first + before[tid];
-        if (blockIdx.x == 0 && tokens_per_expert != nullptr) tokens_per_expert[tid] = total[tid];
-    }
-    if (blockIdx.x == 0) {   // rows that nothing maps to (only if the caller's row count exceeds the set entries)
-        int nnz = 0;
-        for (int e = 0; e < E; ++e) nnz += total[e];
-        for (int r = nnz + tid; r < num_rows; r += 256) sorted_flat[r] = -1;
-    }
-    __syncthreads();
-    // own tokens, in order, one thread per expert column
-    if (tid < E) {
-        int next = base[tid];
-        for (int t = t0; t < t1; ++t) {
-            const int64_t i = static_cast<int64_t>(t) * E + tid;
-            int row = 0x7fffffff;
-            if (map[i] != 0) {
-                if (next < num_rows) {
-                    row = next;
-                    sorted_flat[row] = static_cast<int32_t>(i);
-                }
-                ++next;
-            }
-            row_id_map[i] = row;
-            rows[(t - t0) * E + tid] = row;
-        }
-    }
-    __syncthreads();
-    if (tokens == nullptr) return;
+    const int n = num_tokens * E;
+    const int split = t0 * E;                   // flat entries in front of this workgroup
+    const int own = (t1 - t0) * E;              // this workgroup's entries
     const int local_row = tid / lanes;
     const int lane = tid % lanes;
     const int t = t0 + local_row;
-    if (t >= num_tokens) return;
-    const v16 *src = tokens + static_cast<int64_t>(t) * vecs_per_row;
-    int d[16];
+    const bool mover = tokens != nullptr && t < num_tokens;
+    const v16 *src = tokens + static_cast<int64_t>(mover ? t : 0) * vecs_per_row;
+
+    if (tid < 256) {
 #pragma unroll
-    for (int j = 0; j < 16; ++j) d[j] = j < E ? rows[local_row * E + j] : 0x7fffffff;
-    for (int c0 = lane; c0 < vecs_per_row; c0 += 4 * lanes) {
-        v16 v[4];
+        for (int r = 0; r < 32; ++r) table[r * 256 + tid] = 0;
+    }
+    const int nvec = n / 16;
+    const v16 *mv = reinterpret_cast<const v16 *>(map);
+    v16 w = {0u, 0u, 0u, 0u};
+    if (nvec > 0) w = mv[min(tid, nvec - 1)];
+    unsigned char own0 = 0;
+    if (tid < 64) own0 = map[min(split + tid, n - 1)];
+    v16 v[8];                                   // the first vectors of this thread's row (clamped, unconditional)
+    if (tokens != nullptr) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
-            if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
+        for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+    }
+    __syncthreads();
+    mask_vector_add(table, w, tid * 16, tid < nvec ? 1 : 0, split, E);
+    for (int vi = tid + nthreads; vi < nvec; vi += nthreads) mask_vector_add(table, mv[vi], vi * 16, 1, split, E);
+    for (int i = nvec * 16 + tid; i < n; i += nthreads)     // entries past the last whole vector (small maps only)
+        __hip_atomic_fetch_add(table + ((i < split ? 0 : 16) + (i & (E - 1))) * 256 + (tid & 255), map[i] != 0 ? 1 : 0,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __syncthreads();
+    fused_fold<16>(table, sums);
+    __syncthreads();
+    if (tid < E) {
+        int first = 0;
+        for (int e = 0; e < tid; ++e) first += sums[e] + sums[16 + e];
+        base[tid] = first + sums[tid];
+        if (blockIdx.x == 0 && tokens_per_expert != nullptr) tokens_per_expert[tid] = sums[tid] + sums[16 + tid];
+    }
+    if (blockIdx.x == 0) {   // rows that nothing maps to (only if the caller's row count exceeds the set entries)
+        int nnz = 0;
+        for (int e = 0; e < E; ++e) nnz += sums[e] + sums[16 + e];
+        for (int r = nnz + tid; r < num_rows; r += nthreads) sorted_flat[r] = -1;
+    }
+    __syncthreads();
+    // Own entries in flat order, 64 at a time: lane l always sees expert l % E (E divides 64).  An entry's row
+    // is its expert's next free row plus the set entries of the same expert on lower lanes.
+    if (tid < 64) {
+        const int e = tid & (E - 1);
+        unsigned long long same = 1ull << e;
+        for (int sft = E; sft < 64; sft <<= 1) same |= same << sft;
+        int next = base[e];
+        for (int q0 = 0; q0 < own; q0 += 64) {
+            const int q = q0 + tid;
+            const bool valid = q < own;
+            const unsigned char byte = q0 == 0 ? own0 : (valid ? map[split + q] : 0);
+            const bool set = valid && byte != 0;
+            const unsigned long long mine = __ballot(set) & same;
+            const int rank = next + lanes_below(mine);
+            int row = 0x7fffffff;                // unset or dropped: an id no row count reaches
+            if (set && rank < num_rows) {
+                row = rank;
+                sorted_flat[row] = split + q;
+            }
+            if (valid) {
+                row_id_map[split + q] = row;
+                rows[q] = row;
+            }
+            next += __popcll(mine);
+        }
+    }
+    __syncthreads();
+    if (!mover) return;
+    const int *d = rows + local_row * E;
+    for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
+        if (c0 != lane) {
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            if (static_cast<unsigned>(d[j]) >= static_cast<unsigned>(num_rows)) continue;
-            v16 *dst = permuted + static_cast<int64_t>(d[j]) * vecs_per_row;
+            for (int u = 0; u < 8; ++u)
+                if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
+        }
+        for (int j = 0; j < E; ++j) {
+            const int row = d[j];
+            if (static_cast<unsigned>(row) >= static_cast<unsigned>(num_rows)) continue;
+            v16 *dst = permuted + static_cast<int64_t>(row) * vecs_per_row;
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (int u = 0; u < 8; ++u)
                 if (c0 + u * lanes < vecs_per_row) dst[c0 + u * lanes] = v[u];
         }
     }
@@ -890,12 +1012,26 @@ int launch_permute_fused(hipStream_t stream, const SortPlan &p, const void *toke
                          int64_t T, int64_t k, int64_t row_bytes) {
     const int64_t vecs = row_bytes / sizeof(VecT);
     const RowLayout rl = row_layout(vecs);
-    const int64_t blocks = ceil_div(T, rl.rows_per_block);
-    const size_t lds = (static_cast<size_t>(9) * p.nbins + 16) * sizeof(int);
-    hipLaunchKernelGGL((permute_fused_kernel<IdxT, VecT>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, stream,
-                       static_cast<const VecT *>(tokens), static_cast<VecT *>(permuted), idx, p.n, p.nbins, p.nbits,
-                       num_out, row_id_map, sorted_indices, tpe, tpe_n, static_cast<int>(T), static_cast<int>(k),
-                       static_cast<int>(vecs), rl.lanes);
+    // Fat workgroups repeat the counting less often; keep at least one workgroup per compute unit, and the
+    // workgroup's flat positions within what its LDS hand-over holds.
+    int threads = 1024;
+    while (threads > 256 && (ceil_div(T, threads / rl.lanes) < 256 || (threads / rl.lanes) * k > kFusedMaxLocal))
+        threads >>= 1;
+    const int rows_per_block = threads / rl.lanes;
+    const size_t local = static_cast<size_t>(rows_per_block) * k;
+    if (local > static_cast<size_t>(kFusedMaxLocal)) return -1;   // very short rows with a large top-k: two launches
+    const dim3 grid(static_cast<unsigned>(ceil_div(T, rows_per_block)));
+#define MS_FUSED_ARGS                                                                                                  \
+    static_cast<const VecT *>(tokens), static_cast<VecT *>(permuted), idx, p.n, p.nbins, p.nbits, num_out, row_id_map, \
+        sorted_indices, tpe, tpe_n, static_cast<int>(T), static_cast<int>(k), static_cast<int>(vecs), rl.lanes
+    if (p.nbins <= 8) {
+        const size_t lds = (static_cast<size_t>(16) * 256 + 16 + 8 + local) * sizeof(int);
+        hipLaunchKernelGGL((permute_fused_kernel<IdxT, VecT, 8>), grid, dim3(threads), lds, stream, MS_FUSED_ARGS);
+    } else {
+        const size_t lds = (static_cast<size_t>(32) * 256 + 32 + 16 + local) * sizeof(int);
+        hipLaunchKernelGGL((permute_fused_kernel<IdxT, VecT, 16>), grid, dim3(threads), lds, stream, MS_FUSED_ARGS);
+    }
+#undef MS_FUSED_ARGS
     MS_CHECK_LAUNCH("permute_fused_kernel");
     return MS_OK;
 }
@@ -923,17 +1059,17 @@ int launch_gather_combine(hipStream_t stream, const void *rows, const int32_t *m
     const int64_t vecs = vec_ok ? H / VEC : H;
     const RowLayout rl = row_layout(vecs);
     const unsigned blocks = static_cast<unsigned>(ceil_div(T, rl.rows_per_block));
-    if (vec_ok) {
-        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC>), dim3(blocks), dim3(256), 0, stream,
-                           static_cast<const S *>(rows), map, static_cast<const S *>(probs), static_cast<S *>(out),
-                           static_cast<int>(T), static_cast<int>(k), static_cast<int>(H),
-                           static_cast<int>(num_rows), rl.lanes);
+#define MS_GC_ARGS                                                                                                  \
+    static_cast<const S *>(rows), map, static_cast<const S *>(probs), static_cast<S *>(out), static_cast<int>(T),   \
+        static_cast<int>(k), static_cast<int>(H), static_cast<int>(num_rows), rl.lanes
+    if (!vec_ok) {
+        hipLaunchKernelGGL((gather_combine_kernel<DT, 1, 8, 2>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
+    } else if (k <= 2) {
+        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC, 2, 4>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
     } else {
-        hipLaunchKernelGGL((gather_combine_kernel<DT, 1>), dim3(blocks), dim3(256), 0, stream,
-                           static_cast<const S *>(rows), map, static_cast<const S *>(probs), static_cast<S *>(out),
-                           static_cast<int>(T), static_cast<int>(k), static_cast<int>(H),
-                           static_cast<int>(num_rows), rl.lanes);
+        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC, 8, 2>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
     }
+#undef MS_GC_ARGS
     MS_CHECK_LAUNCH("gather_combine_kernel");
     return MS_OK;
 }
@@ -946,19 +1082,20 @@ int launch_unpermute_grad(hipStream_t stream, const void *permuted, const void *
     constexpr int VEC = 16 / sizeof(S);
     const bool vec_ok = (H % VEC == 0) && aligned16(gy) && aligned16(gperm) && (permuted == nullptr || aligned16(permuted));
     const int64_t vecs = vec_ok ? H / VEC : H;
-    int threads = 64;
-    while (threads < 256 && threads < vecs) threads <<= 1;
-    if (vec_ok) {
-        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC>), dim3(static_cast<unsigned>(T)), dim3(threads), 0, stream,
-                           static_cast<const S *>(permuted), static_cast<const S *>(gy), map,
-                           static_cast<const S *>(probs), static_cast<S *>(gperm), static_cast<S *>(gprobs),
-                           static_cast<int>(k), static_cast<int>(H), static_cast<int>(num_rows));
+    const RowLayout rl = row_layout(vecs);
+    const dim3 grid(static_cast<unsigned>(ceil_div(T, rl.rows_per_block)));
+#define MS_UG_ARGS                                                                                                   \
+    static_cast<const S *>(permuted), static_cast<const S *>(gy), map, static_cast<const S *>(probs),                \
+        static_cast<S *>(gperm), static_cast<S *>(gprobs), static_cast<int>(T), static_cast<int>(k),                 \
+        static_cast<int>(H), static_cast<int>(num_rows), rl.lanes
+    if (!vec_ok) {
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, 1, 4, 4>), grid, dim3(256), 0, stream, MS_UG_ARGS);
+    } else if (k <= 2) {
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC, 2, 4>), grid, dim3(256), 0, stream, MS_UG_ARGS);
     } else {
-        hipLaunchKernelGGL((unpermute_grad_kernel<DT, 1>), dim3(static_cast<unsigned>(T)), dim3(threads), 0, stream,
-                           static_cast<const S *>(permuted), static_cast<const S *>(gy), map,
-                           static_cast<const S *>(probs), static_cast<S *>(gperm), static_cast<S *>(gprobs),
-                           static_cast<int>(k), static_cast<int>(H), static_cast<int>(num_rows));
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC, 4, 2>), grid, dim3(256), 0, stream, MS_UG_ARGS);
     }
+#undef MS_UG_ARGS
     MS_CHECK_LAUNCH("unpermute_grad_kernel");
     return MS_OK;
 }
@@ -1017,12 +1154,15 @@ extern "C" int ms_moe_token_permute(ms_stream_t stream_, const void *tokens, con
     const int64_t row_bytes = H * dtype_size(dtype);
     // small inputs with a known, modest number of experts: sort and row scatter in one launch
     if (p.small && p.nbins <= kFusedMaxBins && num_out > 0) {
-        if (index_dtype == MS_INT32)
-            return permute_fused_dispatch(stream, p, tokens, permuted, static_cast<const int32_t *>(indices), (int)num_out,
-                                          row_id_map, sorted_indices, tokens_per_expert, (int)experts_hint, T, k, row_bytes,
-                                          dtype);
-        return permute_fused_dispatch(stream, p, tokens, permuted, static_cast<const int64_t *>(indices), (int)num_out,
-                                      row_id_map, sorted_indices, tokens_per_expert, (int)experts_hint, T, k, row_bytes, dtype);
+        const int fused =
+            index_dtype == MS_INT32
+                ? permute_fused_dispatch(stream, p, tokens, permuted, static_cast<const int32_t *>(indices), (int)num_out,
+                                         row_id_map, sorted_indices, tokens_per_expert, (int)experts_hint, T, k, row_bytes,
+                                         dtype)
+                : permute_fused_dispatch(stream, p, tokens, permuted, static_cast<const int64_t *>(indices), (int)num_out,
+                                         row_id_map, sorted_indices, tokens_per_expert, (int)experts_hint, T, k, row_bytes,
+                                         dtype);
+        if (fused != -1) return fused;
     }
     int rc;
     if (index_dtype == MS_INT32)
@@ -1136,24 +1276,31 @@ extern "C" int ms_moe_routing_map_permute(ms_stream_t stream_, const void *token
     if (tokens != nullptr)
         if (int rc = check_common(fn, T, E, H, dtype)) return rc;
     if (T == 0) return MS_OK;
-    MS_REQUIRE(routing_map && row_id_map && sorted_flat, MS_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", fn);
+    MS_REQUIRE(routing_map && row_id_map && (sorted_flat || num_rows == 0), MS_ERR_INVALID_ARGUMENT,
+               "%s: NULL tensor pointer", fn);
     MS_REQUIRE(tokens == nullptr || permuted != nullptr || num_rows == 0, MS_ERR_INVALID_ARGUMENT, "%s: permuted is NULL", fn);
     // one launch when whole tokens fit a 16-byte vector of the map and rows move as 16-byte vectors
     const int64_t row_bytes_f = H * dtype_size(dtype);
     const bool pow2 = (E & (E - 1)) == 0 && E <= 16;
-    if (!drop_and_pad && pow2 && aligned16(routing_map) &&
+    if (!drop_and_pad && pow2 && T * E <= kFusedMapMax && aligned16(routing_map) &&
         (tokens == nullptr || (row_bytes_f % 16 == 0 && aligned16(tokens) && aligned16(permuted)))) {
         const int64_t vecs = tokens != nullptr ? row_bytes_f / 16 : 1;
-        const RowLayout rl = tokens != nullptr ? row_layout(vecs) : RowLayout{1, 256};
-        const int64_t blocks = ceil_div(T, rl.rows_per_block);
-        const size_t lds = (48 + static_cast<size_t>(rl.rows_per_block) * E) * sizeof(int);
-        hipLaunchKernelGGL(routing_map_fused_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), lds, stream,
-                           static_cast<const v16 *>(tokens), static_cast<v16 *>(permuted),
-                           static_cast<const unsigned char *>(routing_map), static_cast<int>(T), static_cast<int>(E),
-                           static_cast<int>(num_rows), row_id_map, sorted_flat, tokens_per_expert, static_cast<int>(vecs),
-                           rl.lanes);
-        MS_CHECK_LAUNCH("routing_map_fused_kernel");
-        return MS_OK;
+        const int lanes = tokens != nullptr ? row_layout(vecs).lanes : 1;
+        // fat workgroups repeat the counting less often; keep one per compute unit, and the own entries within
+        // what the LDS hand-over holds
+        int threads = 1024;
+        while (threads > 256 && (ceil_div(T, threads / lanes) < 256 || (threads / lanes) * E > kFusedMaxLocal)) threads >>= 1;
+        const int rows_per_block = threads / lanes;
+        if (static_cast<int64_t>(rows_per_block) * E <= kFusedMaxLocal) {
+            const size_t lds = (static_cast<size_t>(32) * 256 + 48 + static_cast<size_t>(rows_per_block) * E) * sizeof(int);
+            hipLaunchKernelGGL(routing_map_fused_kernel, dim3(static_cast<unsigned>(ceil_div(T, rows_per_block))),
+                               dim3(threads), lds, stream, static_cast<const v16 *>(tokens), static_cast<v16 *>(permuted),
+                               static_cast<const unsigned char *>(routing_map), static_cast<int>(T), static_cast<int>(E),
+                               static_cast<int>(num_rows), row_id_map, sorted_flat, tokens_per_expert,
+                               static_cast<int>(vecs), lanes);
+            MS_CHECK_LAUNCH("routing_map_fused_kernel");
+            return MS_OK;
+        }
     }
     const RoutingPlan r = make_routing_plan(T, E, drop_and_pad);
     MS_REQUIRE(workspace != nullptr && workspace_bytes >= r.total, MS_ERR_WORKSPACE_TOO_SMALL, "%s: workspace %zu < %zu bytes",
@@ -1187,11 +1334,11 @@ extern "C" int ms_moe_routing_map_probs(ms_stream_t stream_, const int32_t *sort
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char *fn = "ms_moe_routing_map_probs";
     MS_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31) && E >= 1, MS_ERR_INVALID_ARGUMENT, "%s: bad sizes", fn);
-    MS_REQUIRE((probs == nullptr) == (permuted_probs == nullptr), MS_ERR_INVALID_ARGUMENT,
-               "%s: probs and permuted_probs must be given together", fn);
     MS_REQUIRE(probs == nullptr || dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED,
                "%s: dtype %d is not one of bf16/fp16/fp32", fn, dtype);
-    if (num_rows == 0) return MS_OK;
+    if (num_rows == 0) return MS_OK;   // empty outputs may come as NULL
+    MS_REQUIRE((probs == nullptr) == (permuted_probs == nullptr), MS_ERR_INVALID_ARGUMENT,
+               "%s: probs and permuted_probs must be given together", fn);
     MS_REQUIRE(sorted_flat != nullptr, MS_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", fn);
     const dim3 grid(static_cast<unsigned>(ceil_div(num_rows, 256)));
     // a probability is only moved, never computed with: 2-byte types share one instantiation

@@ -90,6 +90,38 @@ def test_permute_empty_and_negative_num_out(device):
     assert e_perm.shape == (0, 8) and e_map.numel() == 0
 
 
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+@pytest.mark.parametrize("T,E", [(300, 8), (4096, 8), (1000, 16), (700, 200)])
+def test_permute_out_of_range_ids_are_clamped(idt, T, E, device):
+    """Expert ids outside [0, num_experts) are clamped into range before sorting (negative ones to the first
+    expert, large ones to the last bin), for every index width, also when only the upper half of a 64-bit id is
+    set.  The bins are a power of two, so ids up to the next power of two keep their own bin."""
+    say("permute clamp case", idt, T, E)
+    k, H = 2, 64
+    gen = torch.Generator().manual_seed(T + E)
+    idx = torch.randint(0, E, (T, k), generator=gen).to(idt)
+    nbins = 2
+    while nbins < E:
+        nbins *= 2
+    odd = [-1, -7, nbins, nbins + 100, 2 ** 31 - 1]
+    if idt == torch.int64:
+        odd += [2 ** 33 + 3, -(2 ** 40), 2 ** 62]
+    where = torch.randperm(T * k, generator=gen)[:len(odd) * 3]
+    flat = idx.view(-1)
+    for i, pos in enumerate(where.tolist()):
+        flat[pos] = odd[i % len(odd)]
+    clamped = idx.clamp(0, nbins - 1)
+    tokens = torch.randn(T, H, generator=gen).to(torch.bfloat16)
+    exp_perm, exp_map = O.fused_permute(tokens, clamped, None)
+    _, exp_sorted = O.permute(tokens, clamped, exp_perm.size(0))
+    perm, rmap, srt, counts = ops.moe_token_permute_with_aux(tokens.to(device), idx.to(device), None, num_experts=E)
+    torch.cuda.synchronize()
+    assert torch.equal(rmap.cpu(), exp_map)
+    assert torch.equal(srt.cpu().long(), exp_sorted)
+    assert torch.equal(perm.cpu(), exp_perm)
+    assert torch.equal(counts.cpu(), torch.bincount(clamped.reshape(-1).long(), minlength=nbins)[:E])
+
+
 UNPERMUTE_CASES = [
     (512, 2, 8, 256, torch.float32, None),
     (300, 4, 16, 136, torch.bfloat16, None),

@@ -186,6 +186,20 @@ def test_full_size_properties(device):
     assert torch.equal(back, tok_d)
 
 
+@pytest.mark.parametrize("T,E", [(5, 4), (1, 32), (300, 7)])
+def test_no_entry_set(T, E, device):
+    """A map with no entry set: zero rows out; unpermute hands an empty input straight back, like the
+    reference does (mindspeed/te/pytorch/permutation.py:81-83)."""
+    say("routing-map empty case", T, E)
+    rmap = torch.zeros(T, E, dtype=torch.bool, device=device)
+    tokens = torch.randn(T, 16, device=device)
+    probs = torch.zeros(T, E, device=device)
+    perm, pp, sidx = M.permute(tokens, rmap, probs, fused=True)
+    assert perm.shape == (0, 16) and pp.numel() == 0 and sidx.numel() == 0
+    back = M.unpermute(perm, sidx, tokens.shape, probs=probs, routing_map=rmap, fused=True)
+    assert back.numel() == 0
+
+
 def test_argument_checks(device):
     tokens = torch.randn(4, 8, device=device)
     rmap = torch.ones(4, 2, dtype=torch.bool, device=device)
