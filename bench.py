@@ -290,6 +290,14 @@ def main():
         torch.cuda.synchronize()
         result["copy_calibration_bytes"] = n
     result["routing_map_mode"] = measure_routing_map_mode(cfg, device, x.detach(), idx, p.detach())
+    # The permute / unpermute family by itself at this workload's shape: back-to-back launches through the C ABI
+    # on resident buffers (the per-op figures under "kernels" are single launches inside the layer step, bracketed
+    # by events, i.e. with the launch gaps on either side).  Not part of `value`.
+    from mindspeed_amd.permute_microbench import measure as measure_permute_family
+    result["permute_family"] = {
+        "note": "back-to-back launches through the C ABI, event-timed over 200 launches per op; "
+                "algorithmic bytes over the average, against the 8 TB/s HBM peak",
+        **measure_permute_family(cfg["T"], cfg["H"], cfg["E"], cfg["K"], torch.bfloat16, device=device)}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(result))

@@ -738,7 +738,7 @@ __global__ __launch_bounds__(1024) void permute_fused_kernel(
             VecT *dst = permuted + static_cast<int64_t>(row) * vecs_per_row;
 #pragma unroll
             for (int u = 0; u < 8; ++u)
-                if (c0 + u * lanes < vecs_per_row) dst[c0 + u * lanes] = v[u];
+                if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + c0 + u * lanes);
         }
     }
 }
@@ -930,7 +930,7 @@ __global__ __launch_bounds__(1024) void routing_map_fused_kernel(
             v16 *dst = permuted + static_cast<int64_t>(row) * vecs_per_row;
 #pragma unroll
             for (int u = 0; u < 8; ++u)
-                if (c0 + u * lanes < vecs_per_row) dst[c0 + u * lanes] = v[u];
+                if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + c0 + u * lanes);
         }
     }
 }

@@ -1,0 +1,119 @@
+"""The permute / unpermute family in isolation: back-to-back launches through the C ABI.
+
+    python -m mindspeed_amd.permute_microbench [--tokens 4096] [--hidden 4096] [--experts 8] [--topk 2]
+                                               [--iters 200] [--warmup 20]
+
+Every op is launched ``--iters`` times in a row on resident buffers (no allocation, no Python op wrapper in
+the loop: one ctypes call per launch, which is shorter than the kernels at the default size) between two
+events on the launch stream, so the average is the kernel's duration plus the gap between launches.  Rates are
+the algorithmic bytes of the op (rows read once and written once, plus its index and probability arrays)
+over that average, next to the 8 TB/s HBM peak.  The ops:
+
+    permute         ms_moe_token_permute          sort by expert + row scatter (expert count given)
+    permute_mask    ms_moe_routing_map_permute    the same from a [tokens, experts] boolean map
+    unpermute       ms_moe_token_unpermute        probability-weighted top-k gather
+    unpermute_grad  ms_moe_token_unpermute_grad   grad of rows and of probabilities
+    permute_grad    ms_moe_token_permute_grad     unweighted top-k gather
+    copy            ms_copy_bytes                 plain copy of the permuted rows, for orientation
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+
+import torch
+
+from . import _lib, flop_counter
+
+HBM_PEAK_GBS = 8000.0
+
+
+def measure(num_tokens=4096, hidden=4096, num_experts=8, topk=2, dtype=torch.bfloat16, iters=200, warmup=20,
+            device=None):
+    """Returns ``{op: {"avg_us", "gbs", "bytes_per_launch", "frac_of_hbm_peak"}}`` for the ops listed above."""
+    if not torch.cuda.is_available():
+        raise RuntimeError("permute_microbench needs a HIP device")
+    dev = torch.device("cuda", 0) if device is None else device
+    lib = _lib.load()
+    T, H, E, K = num_tokens, hidden, num_experts, topk
+    elem = torch.empty(0, dtype=dtype).element_size()
+    code = _lib.dtype_code(dtype, "tokens")
+    gen = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(T, H, generator=gen, device=dev).to(dtype)
+    idx = torch.topk(torch.randn(T, E, generator=gen, device=dev), K, dim=-1)[1].contiguous()   # int64, distinct per token
+    probs = torch.rand(T, K, generator=gen, device=dev).to(dtype)
+    gy = torch.randn(T, H, generator=gen, device=dev).to(dtype)
+    rmap = torch.zeros(T, E, dtype=torch.bool, device=dev)
+    rmap.scatter_(1, idx, True)
+    rows = T * K
+    perm = torch.empty(rows, H, dtype=dtype, device=dev)
+    row_id_map = torch.empty(rows, dtype=torch.int32, device=dev)
+    sorted_idx = torch.empty(rows, dtype=torch.int32, device=dev)
+    counts = torch.empty(E, dtype=torch.int64, device=dev)
+    mask_map = torch.empty(T * E, dtype=torch.int32, device=dev)
+    mask_sorted = torch.empty(rows, dtype=torch.int32, device=dev)
+    out = torch.empty(T, H, dtype=dtype, device=dev)
+    gperm = torch.empty_like(perm)
+    gprobs = torch.empty_like(probs)
+    copy_dst = torch.empty_like(perm)
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(lib.ms_moe_token_permute_workspace_size(T, K, E, ctypes.byref(nbytes)), "workspace_size")
+    ws = _lib.workspace(nbytes.value, dev)
+    _lib.check(lib.ms_moe_routing_map_workspace_size(T, E, 0, ctypes.byref(nbytes)), "workspace_size")
+    ws_mask = _lib.workspace(nbytes.value, dev)
+    stream = _lib.stream_ptr(dev)
+    P = _lib.ptr
+
+    ops = {
+        "permute": (lambda: lib.ms_moe_token_permute(
+            stream, P(x), P(idx), _lib.MS_INT64, T, K, H, code, rows, E, P(perm), P(row_id_map), P(sorted_idx),
+            P(counts), P(ws), ws.numel()), flop_counter.permute_bytes(T, K, H, elem, 8)),
+        "permute_mask": (lambda: lib.ms_moe_routing_map_permute(
+            stream, P(x), P(rmap), T, E, H, code, rows, 0, P(perm), P(mask_map), P(mask_sorted), P(counts),
+            P(ws_mask), ws_mask.numel()), T * H * elem + rows * H * elem + T * E * (1 + 4) + rows * 4),
+        "unpermute": (lambda: lib.ms_moe_token_unpermute(
+            stream, P(perm), P(row_id_map), P(probs), T, K, H, code, rows, P(out)),
+            flop_counter.unpermute_bytes(T, K, H, elem)),
+        "unpermute_grad": (lambda: lib.ms_moe_token_unpermute_grad(
+            stream, P(perm), P(gy), P(row_id_map), P(probs), T, K, H, code, rows, P(gperm), P(gprobs)),
+            flop_counter.unpermute_grad_bytes(T, K, H, elem)),
+        "permute_grad": (lambda: lib.ms_moe_token_permute_grad(
+            stream, P(perm), P(row_id_map), T, K, H, code, rows, P(out)), flop_counter.permute_grad_bytes(T, K, H, elem)),
+        "copy": (lambda: lib.ms_copy_bytes(stream, P(perm), P(copy_dst), perm.numel() * elem), 2 * perm.numel() * elem),
+    }
+    result = {}
+    with torch.cuda.device(dev):
+        for name, (launch, work) in ops.items():   # "permute" runs first: the later ops read its outputs
+            for _ in range(warmup):
+                _lib.check(launch(), name)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                launch()
+            e1.record()
+            torch.cuda.synchronize(dev)
+            us = e0.elapsed_time(e1) * 1e3 / iters
+            gbs = work / us / 1e3
+            result[name] = {"avg_us": round(us, 2), "gbs": round(gbs, 1), "bytes_per_launch": int(work),
+                            "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+    return result
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--tokens", type=int, default=4096)
+    ap.add_argument("--hidden", type=int, default=4096)
+    ap.add_argument("--experts", type=int, default=8)
+    ap.add_argument("--topk", type=int, default=2)
+    ap.add_argument("--iters", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    a = ap.parse_args()
+    res = measure(a.tokens, a.hidden, a.experts, a.topk, torch.bfloat16, a.iters, a.warmup)
+    print(f"{a.tokens} tokens x hidden {a.hidden}, {a.experts} experts, top-{a.topk}, bf16; {a.iters} launches per op")
+    for name, r in res.items():
+        print(f"{name:15s} {r['avg_us']:8.2f} us  {r['gbs']:8.1f} GB/s  {r['frac_of_hbm_peak']:.3f} of 8 TB/s  "
+              f"({r['bytes_per_launch'] / 1e6:.1f} MB per launch)", flush=True)
+
+
+if __name__ == "__main__":
+    main()
