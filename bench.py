@@ -222,6 +222,17 @@ def main():
         torch.cuda.synchronize()
         ms_per_step_events = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # what an empty bracket reads: the per-op times below include this much that is not the kernel
+    stream = torch.cuda.current_stream(device)
+    pairs = []
+    for _ in range(50):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        e1.record(stream)
+        pairs.append((e0, e1))
+    torch.cuda.synchronize()
+    empty_bracket_ms = sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
+
     kernels = {}
     for name, s in rec.summary().items():
         avg_ms = s["ms"] / s["calls"]
@@ -278,6 +289,8 @@ def main():
                                                                                   * cfg["H"] * cfg["F"] / 1e12, 3)},
         "roofline": roofline,
         "kernels": kernels,
+        "kernels_note": "single launches inside the layer step, each between two events on its stream; an empty "
+                        f"bracket reads {empty_bracket_ms * 1e3:.1f} us on this box",
     }
     if args.copy_calibration:
         from mindspeed_amd import _lib
