@@ -591,6 +591,7 @@ __device__ __forceinline__ int fused_key(int64_t raw, int last, unsigned &bad) {
     }
 }
 
+constexpr int kScanInKernelMax = 16384;  // histogram entries (segments x bins) a scatter workgroup adds up itself
 constexpr int kFusedKeys = 8;         // keys per thread in flight at a time
 
 // One batch of raw indices: flat positions c + u * blockDim.x + tid.
@@ -724,6 +725,226 @@ __global__ __launch_bounds__(1024) void permute_fused_kernel(
     }
     __syncthreads();
 
+    if (!mover) return;
+    const int *d = dest + local_row * topk;
+    for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
+        if (c0 != lane) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
+        }
+        for (int j = 0; j < topk; ++j) {
+            const int row = d[j];
+            if (static_cast<unsigned>(row) >= static_cast<unsigned>(num_out)) continue;   // dropped
+            VecT *dst = permuted + static_cast<int64_t>(row) * vecs_per_row;
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + c0 + u * lanes);
+        }
+    }
+}
+
+// The one-launch permute for more than kFusedMaxBins bins (up to MS_MAX_EXPERTS, which is what a call without
+// an expert count sorts into) and n <= kSmallSortMax.  Same scheme as permute_fused_kernel, but the counters are
+// one LDS word per bin and per side (in front of the workgroup's first position / all), added to directly: with
+// many bins the lanes of an instruction rarely meet on a word, and a table of private columns would not fit.
+template <typename IdxT, typename VecT>
+__global__ __launch_bounds__(1024) void permute_fused_bins_kernel(
+    const VecT *__restrict__ tokens, VecT *__restrict__ permuted, const IdxT *__restrict__ idx, int n, int nbins,
+    int nbits, int num_out, int32_t *__restrict__ row_id_map, int32_t *__restrict__ sorted_indices,
+    int64_t *__restrict__ tokens_per_expert, int tpe_n, int num_tokens, int topk, int vecs_per_row, int lanes) {
+    extern __shared__ int lds[];               // bef[nbins], tot[nbins], scratch[32], dest[rows_per_block * topk]
+    int *bef = lds;
+    int *tot = lds + nbins;
+    int *scratch = tot + nbins;
+    int *dest = scratch + 32;
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    const int rows_per_block = nthreads / lanes;
+    const int t0 = blockIdx.x * rows_per_block;
+    const int t1 = min(t0 + rows_per_block, num_tokens);
+    const int p0 = t0 * topk, p1 = t1 * topk;  // this workgroup's flat positions
+    const int local_row = tid / lanes;
+    const int lane = tid % lanes;
+    const int t = t0 + local_row;
+    const bool mover = t < num_tokens;
+    const VecT *src = tokens + static_cast<int64_t>(mover ? t : 0) * vecs_per_row;
+
+    for (int e = tid; e < 2 * nbins; e += nthreads) lds[e] = 0;
+    IdxT raw[kFusedKeys];
+    fused_load(raw, idx, 0, n);
+    const bool few_own = p1 - p0 <= 64;
+    IdxT own = 0;
+    if (tid < 64) own = idx[min(p0 + tid, n - 1)];
+    VecT v[8];   // first vectors of this thread's row: unconditional loads from clamped positions, in flight
+                 // while the keys are counted
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+    __syncthreads();
+    unsigned unused = 0;
+    for (int c = 0; c < n; c += kFusedKeys * nthreads) {
+        if (c != 0) fused_load(raw, idx, c, n);
+#pragma unroll
+        for (int u = 0; u < kFusedKeys; ++u) {
+            const int pos = c + u * nthreads + tid;
+            const int key = fused_key<true>(raw[u], nbins - 1, unused);
+            __hip_atomic_fetch_add(tot + key, pos < n ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __hip_atomic_fetch_add(bef + key, pos < p0 ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    }
+    __syncthreads();
+    // bins in passes of one per thread, the running row count carried from pass to pass; bef[bin] becomes the
+    // bin's next free row as seen from this workgroup
+    int carry = 0;
+    for (int e0 = 0; e0 < nbins; e0 += nthreads) {
+        const int bin = e0 + tid;
+        const int total = bin < nbins ? tot[bin] : 0;
+        const int first = carry + block_exclusive_scan(total, scratch);
+        if (bin < nbins) {
+            bef[bin] += first;
+            if (blockIdx.x == 0 && tokens_per_expert != nullptr && bin < tpe_n) tokens_per_expert[bin] = total;
+        }
+        if (tid == nthreads - 1) scratch[16] = first + total;
+        __syncthreads();
+        carry = scratch[16];
+        __syncthreads();
+    }
+    if (tid < 64) {
+        if (few_own) {
+            int keys[kKeysPerLane];
+#pragma unroll
+            for (int u = 1; u < kKeysPerLane; ++u) keys[u] = -1;
+            keys[0] = p0 + tid < p1 ? fused_key<true>(own, nbins - 1, unused) : -1;
+            scatter_chunk(bef, keys, p0, p1 - p0, nbins, nbits, num_out, row_id_map, sorted_indices, dest, p0);
+        } else {
+            wave_scatter(bef, idx, p0, p1, nbins, nbits, num_out, row_id_map, sorted_indices, dest);
+        }
+    }
+    __syncthreads();
+    if (!mover) return;
+    const int *d = dest + local_row * topk;
+    for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
+        if (c0 != lane) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
+        }
+        for (int j = 0; j < topk; ++j) {
+            const int row = d[j];
+            if (static_cast<unsigned>(row) >= static_cast<unsigned>(num_out)) continue;   // dropped
+            VecT *dst = permuted + static_cast<int64_t>(row) * vecs_per_row;
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + c0 + u * lanes);
+        }
+    }
+}
+
+// Stable scatter and row movement in one launch, behind the histogram launch of the multi-block sort (any bin
+// count, any number of positions).  A workgroup ranks its own flat positions.  For the segment its first
+// position lies in it needs, per bin, the first row of that (segment, bin):
+//   SCANNED = true:  table[s][bin] holds it (sort_scan_kernel has run);
+//   SCANNED = false: table[s][bin] is still the segment's histogram, and the workgroup adds up, per bin, all
+//                    segments (-> first row of the bin, after a scan over the bins) and the segments in front of
+//                    its own; the host picks this form while the table is small enough to read per workgroup.
+// To that it adds the keys of its segment in front of its first position, counted by all threads with LDS adds,
+// and its first wavefront runs the same stable scatter as sort_scatter_kernel over the workgroup's positions,
+// piece by piece where they cross a segment boundary.  The rows reach the copying threads through LDS; the
+// first vectors of the source rows are requested before the counting.
+template <typename IdxT, typename VecT, bool SCANNED>
+__global__ __launch_bounds__(1024) void permute_scatter_rows_kernel(
+    const VecT *__restrict__ tokens, VecT *__restrict__ permuted, const IdxT *__restrict__ idx, int n, int seg, int nseg,
+    int nbins, int nbits, const int *__restrict__ table, int num_out, int32_t *__restrict__ row_id_map,
+    int32_t *__restrict__ sorted_indices, int64_t *__restrict__ tokens_per_expert, int tpe_n, int num_tokens, int topk,
+    int vecs_per_row, int lanes) {
+    extern __shared__ int lds[];               // cnt[nbins], first[nbins], pre[nbins], scratch[32], dest[rows_per_block * topk]
+    int *cnt = lds;
+    int *first = lds + nbins;
+    int *pre = first + nbins;
+    int *scratch = pre + nbins;
+    int *dest = scratch + 32;
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    const int rows_per_block = nthreads / lanes;
+    const int t0 = blockIdx.x * rows_per_block;
+    const int t1 = min(t0 + rows_per_block, num_tokens);
+    const int p0 = t0 * topk, p1 = t1 * topk;  // this workgroup's flat positions
+    const int local_row = tid / lanes;
+    const int lane = tid % lanes;
+    const int t = t0 + local_row;
+    const bool mover = t < num_tokens;
+    const VecT *src = tokens + static_cast<int64_t>(mover ? t : 0) * vecs_per_row;
+    const int s0 = p0 / seg;
+    const int seg_begin = s0 * seg;
+
+    for (int e = tid; e < 3 * nbins; e += nthreads) lds[e] = 0;
+    constexpr int KU = 4;
+    IdxT raw[KU];
+#pragma unroll
+    for (int u = 0; u < KU; ++u) raw[u] = idx[min(seg_begin + u * nthreads + tid, n - 1)];
+    VecT v[8];   // first vectors of this thread's row: unconditional loads from clamped positions, in flight
+                 // while the keys above are counted
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+    __syncthreads();
+    for (int c = seg_begin; c < p0; c += KU * nthreads) {
+        if (c != seg_begin) {
+#pragma unroll
+            for (int u = 0; u < KU; ++u) raw[u] = idx[min(c + u * nthreads + tid, n - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < KU; ++u) {
+            long long key = static_cast<long long>(raw[u]);
+            key = key < 0 ? 0 : key;
+            key = key >= nbins ? nbins - 1 : key;
+            if (c + u * nthreads + tid < p0) atomicAdd(&cnt[static_cast<int>(key)], 1);
+        }
+    }
+    if constexpr (!SCANNED) {
+        for (int i = tid; i < nseg * nbins; i += nthreads) {
+            const int sg = i / nbins;
+            const int e = i - sg * nbins;
+            const int c = table[i];
+            atomicAdd(&first[e], c);                 // per-bin total for now
+            if (sg < s0) atomicAdd(&pre[e], c);
+        }
+        __syncthreads();
+        int carry = 0;
+        for (int e0 = 0; e0 < nbins; e0 += nthreads) {
+            const int bin = e0 + tid;
+            const int total = bin < nbins ? first[bin] : 0;
+            const int start = carry + block_exclusive_scan(total, scratch);
+            if (bin < nbins) {
+                first[bin] = start;
+                if (blockIdx.x == 0 && tokens_per_expert != nullptr && bin < tpe_n) tokens_per_expert[bin] = total;
+            }
+            if (tid == nthreads - 1) scratch[16] = start + total;
+            __syncthreads();
+            carry = scratch[16];
+            __syncthreads();
+        }
+    } else {
+        __syncthreads();
+    }
+    if (tid < 64) {
+        int begin = p0;
+        for (int sgm = s0; begin < p1; ++sgm) {
+            const int end = min(p1, (sgm + 1) * seg);
+            for (int e = tid; e < nbins; e += 64) {
+                if constexpr (SCANNED) {
+                    cnt[e] = table[static_cast<int64_t>(sgm) * nbins + e] + (sgm == s0 ? cnt[e] : 0);
+                } else {
+                    if (sgm != s0) pre[e] += table[static_cast<int64_t>(sgm - 1) * nbins + e];
+                    cnt[e] = first[e] + pre[e] + (sgm == s0 ? cnt[e] : 0);
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+            wave_scatter(cnt, idx, begin, end, nbins, nbits, num_out, row_id_map, sorted_indices, dest + (begin - p0));
+            __builtin_amdgcn_wave_barrier();
+            begin = end;
+        }
+    }
+    __syncthreads();
     if (!mover) return;
     const int *d = dest + local_row * topk;
     for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
@@ -959,6 +1180,22 @@ inline SortPlan make_sort_plan(int64_t n, int64_t experts_hint) {
     return p;
 }
 
+// Histogram launch of the multi-block sort (table[s][bin] = keys of `bin` in segment s) and, with `scan`, the scan
+// launch behind it (table[s][bin] = first row of `bin` for segment s).
+template <typename IdxT>
+int launch_sort_offsets(hipStream_t stream, const SortPlan &p, const IdxT *idx, int64_t *tpe, int tpe_n, int *table,
+                        bool scan = true) {
+    const int blocks = static_cast<int>(ceil_div(p.nseg, kHistWavesPerBlock));
+    const size_t lds = static_cast<size_t>(kHistWavesPerBlock) * p.nbins * sizeof(int);
+    hipLaunchKernelGGL(sort_hist_kernel<IdxT>, dim3(blocks), dim3(kHistWavesPerBlock * 64), lds, stream, idx, p.n,
+                       p.seg, p.nseg, p.nbins, p.nbits, table);
+    MS_CHECK_LAUNCH("sort_hist_kernel");
+    if (!scan) return MS_OK;
+    hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(1024), 0, stream, table, p.nseg, p.nbins, tpe, tpe_n);
+    MS_CHECK_LAUNCH("sort_scan_kernel");
+    return MS_OK;
+}
+
 template <typename IdxT>
 int launch_sort(hipStream_t stream, const SortPlan &p, const IdxT *idx, int num_out, int32_t *row_id_map,
                 int32_t *sorted_indices, int64_t *tpe, int tpe_n, void *workspace) {
@@ -980,13 +1217,9 @@ int launch_sort(hipStream_t stream, const SortPlan &p, const IdxT *idx, int num_
         return MS_OK;
     }
     int *table = static_cast<int *>(workspace);
+    if (int rc = launch_sort_offsets(stream, p, idx, tpe, tpe_n, table)) return rc;
     const int blocks = static_cast<int>(ceil_div(p.nseg, kHistWavesPerBlock));
     const size_t lds = static_cast<size_t>(kHistWavesPerBlock) * p.nbins * sizeof(int);
-    hipLaunchKernelGGL(sort_hist_kernel<IdxT>, dim3(blocks), dim3(kHistWavesPerBlock * 64), lds, stream, idx, p.n,
-                       p.seg, p.nseg, p.nbins, p.nbits, table);
-    MS_CHECK_LAUNCH("sort_hist_kernel");
-    hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(1024), 0, stream, table, p.nseg, p.nbins, tpe, tpe_n);
-    MS_CHECK_LAUNCH("sort_scan_kernel");
     hipLaunchKernelGGL(sort_scatter_kernel<IdxT>, dim3(blocks), dim3(kHistWavesPerBlock * 64), lds, stream, idx,
                        p.n, p.seg, p.nseg, p.nbins, p.nbits, table, num_out, row_id_map, sorted_indices);
     MS_CHECK_LAUNCH("sort_scatter_kernel");
@@ -1024,7 +1257,10 @@ int launch_permute_fused(hipStream_t stream, const SortPlan &p, const void *toke
 #define MS_FUSED_ARGS                                                                                                  \
     static_cast<const VecT *>(tokens), static_cast<VecT *>(permuted), idx, p.n, p.nbins, p.nbits, num_out, row_id_map, \
         sorted_indices, tpe, tpe_n, static_cast<int>(T), static_cast<int>(k), static_cast<int>(vecs), rl.lanes
-    if (p.nbins <= 8) {
+    if (p.nbins > kFusedMaxBins) {
+        const size_t lds = (static_cast<size_t>(2) * p.nbins + 32 + local) * sizeof(int);
+        hipLaunchKernelGGL((permute_fused_bins_kernel<IdxT, VecT>), grid, dim3(threads), lds, stream, MS_FUSED_ARGS);
+    } else if (p.nbins <= 8) {
         const size_t lds = (static_cast<size_t>(16) * 256 + 16 + 8 + local) * sizeof(int);
         hipLaunchKernelGGL((permute_fused_kernel<IdxT, VecT, 8>), grid, dim3(threads), lds, stream, MS_FUSED_ARGS);
     } else {
@@ -1034,6 +1270,52 @@ int launch_permute_fused(hipStream_t stream, const SortPlan &p, const void *toke
 #undef MS_FUSED_ARGS
     MS_CHECK_LAUNCH("permute_fused_kernel");
     return MS_OK;
+}
+
+// Histogram, scan, then scatter + row movement in one launch.  Returns -1 when a workgroup's positions do not
+// fit the LDS hand-over (very short rows with a large top-k).
+template <typename IdxT, typename VecT>
+int launch_permute_scatter_rows(hipStream_t stream, const SortPlan &p, const void *tokens, void *permuted, const IdxT *idx,
+                                int num_out, int32_t *row_id_map, int32_t *sorted_indices, int64_t *tpe, int tpe_n,
+                                int64_t T, int64_t k, int64_t row_bytes, int *table) {
+    const int64_t vecs = row_bytes / sizeof(VecT);
+    const RowLayout rl = row_layout(vecs);
+    int threads = 1024;
+    while (threads > 256 && (ceil_div(T, threads / rl.lanes) < 256 || (threads / rl.lanes) * k > kFusedMaxLocal))
+        threads >>= 1;
+    const int rows_per_block = threads / rl.lanes;
+    const size_t local = static_cast<size_t>(rows_per_block) * k;
+    if (local > static_cast<size_t>(kFusedMaxLocal)) return -1;
+    // a small table is summed by every scatter workgroup itself; a large one gets its own scan launch
+    const bool scan_launch = static_cast<int64_t>(p.nseg) * p.nbins > kScanInKernelMax;
+    if (int rc = launch_sort_offsets(stream, p, idx, tpe, tpe_n, table, scan_launch)) return rc;
+    const size_t lds = (static_cast<size_t>(3) * p.nbins + 32 + local) * sizeof(int);
+    const dim3 grid(static_cast<unsigned>(ceil_div(T, rows_per_block)));
+#define MS_SR_ARGS                                                                                                    \
+    static_cast<const VecT *>(tokens), static_cast<VecT *>(permuted), idx, p.n, p.seg, p.nseg, p.nbins, p.nbits, table, \
+        num_out, row_id_map, sorted_indices, tpe, tpe_n, static_cast<int>(T), static_cast<int>(k),                     \
+        static_cast<int>(vecs), rl.lanes
+    if (scan_launch)
+        hipLaunchKernelGGL((permute_scatter_rows_kernel<IdxT, VecT, true>), grid, dim3(threads), lds, stream, MS_SR_ARGS);
+    else
+        hipLaunchKernelGGL((permute_scatter_rows_kernel<IdxT, VecT, false>), grid, dim3(threads), lds, stream, MS_SR_ARGS);
+#undef MS_SR_ARGS
+    MS_CHECK_LAUNCH("permute_scatter_rows_kernel");
+    return MS_OK;
+}
+
+template <typename IdxT>
+int permute_scatter_rows_dispatch(hipStream_t stream, const SortPlan &p, const void *tokens, void *permuted,
+                                  const IdxT *idx, int num_out, int32_t *row_id_map, int32_t *sorted_indices, int64_t *tpe,
+                                  int tpe_n, int64_t T, int64_t k, int64_t row_bytes, int dtype, int *table) {
+    if (row_bytes % 16 == 0 && aligned16(tokens) && aligned16(permuted))
+        return launch_permute_scatter_rows<IdxT, v16>(stream, p, tokens, permuted, idx, num_out, row_id_map,
+                                                      sorted_indices, tpe, tpe_n, T, k, row_bytes, table);
+    if (dtype == MS_FP32)
+        return launch_permute_scatter_rows<IdxT, uint32_t>(stream, p, tokens, permuted, idx, num_out, row_id_map,
+                                                           sorted_indices, tpe, tpe_n, T, k, row_bytes, table);
+    return launch_permute_scatter_rows<IdxT, uint16_t>(stream, p, tokens, permuted, idx, num_out, row_id_map,
+                                                       sorted_indices, tpe, tpe_n, T, k, row_bytes, table);
 }
 
 template <typename IdxT>
@@ -1125,7 +1407,7 @@ extern "C" int ms_moe_token_permute_workspace_size(int64_t num_tokens, int64_t t
                "ms_moe_token_permute_workspace_size: num_experts_hint %lld exceeds %d", (long long)num_experts_hint,
                MS_MAX_EXPERTS);
     const SortPlan p = make_sort_plan(num_tokens * topk, num_experts_hint);
-    *bytes = p.small ? 0 : static_cast<size_t>(p.nseg) * p.nbins * sizeof(int);
+    *bytes = static_cast<size_t>(p.nseg) * p.nbins * sizeof(int);
     return MS_OK;
 }
 
@@ -1148,12 +1430,12 @@ extern "C" int ms_moe_token_permute(ms_stream_t stream_, const void *tokens, con
     MS_REQUIRE(tokens && indices && row_id_map && (permuted || num_out == 0), MS_ERR_INVALID_ARGUMENT,
                "ms_moe_token_permute: NULL tensor pointer");
     const SortPlan p = make_sort_plan(T * k, experts_hint);
-    const size_t need = p.small ? 0 : static_cast<size_t>(p.nseg) * p.nbins * sizeof(int);
+    const size_t need = static_cast<size_t>(p.nseg) * p.nbins * sizeof(int);
     MS_REQUIRE(workspace_bytes >= need && (need == 0 || workspace != nullptr), MS_ERR_WORKSPACE_TOO_SMALL,
                "ms_moe_token_permute: workspace %zu < %zu bytes", workspace_bytes, need);
     const int64_t row_bytes = H * dtype_size(dtype);
-    // small inputs with a known, modest number of experts: sort and row scatter in one launch
-    if (p.small && p.nbins <= kFusedMaxBins && num_out > 0) {
+    // inputs one workgroup can count: sort and row scatter in one launch
+    if (p.small && num_out > 0) {
         const int fused =
             index_dtype == MS_INT32
                 ? permute_fused_dispatch(stream, p, tokens, permuted, static_cast<const int32_t *>(indices), (int)num_out,
@@ -1163,6 +1445,19 @@ extern "C" int ms_moe_token_permute(ms_stream_t stream_, const void *tokens, con
                                          row_id_map, sorted_indices, tokens_per_expert, (int)experts_hint, T, k, row_bytes,
                                          dtype);
         if (fused != -1) return fused;
+    }
+    // otherwise: histogram and scan launches, then scatter and row movement in one launch
+    if (num_out > 0 && !p.small) {
+        int *table = static_cast<int *>(workspace);
+        const int three =
+            index_dtype == MS_INT32
+                ? permute_scatter_rows_dispatch(stream, p, tokens, permuted, static_cast<const int32_t *>(indices),
+                                                (int)num_out, row_id_map, sorted_indices, tokens_per_expert,
+                                                (int)experts_hint, T, k, row_bytes, dtype, table)
+                : permute_scatter_rows_dispatch(stream, p, tokens, permuted, static_cast<const int64_t *>(indices),
+                                                (int)num_out, row_id_map, sorted_indices, tokens_per_expert,
+                                                (int)experts_hint, T, k, row_bytes, dtype, table);
+        if (three != -1) return three;
     }
     int rc;
     if (index_dtype == MS_INT32)

@@ -42,6 +42,15 @@ PERMUTE_CASES = [
     (8192, 8, 64, 64, torch.bfloat16, torch.int64, None, 64),      # R=65536: multi-block sort
     (5000, 7, 100, 16, torch.bfloat16, torch.int32, 30000, None),  # ragged, drop, 1024 bins
     (1, 8, 256, 32, torch.bfloat16, torch.int64, None, 256),
+    # one launch with per-bin LDS counters (more than 16 bins, R <= 16384)
+    (4096, 2, 8, 1024, torch.bfloat16, torch.int64, None, None),   # 1024 bins, 1024-thread workgroups
+    (700, 6, 60, 96, torch.float16, torch.int32, 3000, 60),        # 64 bins, drop, top-6
+    (2048, 8, 256, 40, torch.float32, torch.int64, None, 256),     # R=16384, 256 bins, 10 lanes per row
+    # histogram launch + scatter/rows launch (R > 16384): table summed per workgroup / by its own scan launch
+    (4099, 6, 12, 128, torch.bfloat16, torch.int64, None, 12),     # top-6: workgroups straddle segment boundaries
+    (3000, 7, 130, 264, torch.bfloat16, torch.int32, 20000, 130),  # 256 bins x 21 segments, drop
+    (9000, 4, 40, 32, torch.float32, torch.int64, None, None),     # 1024 bins x 36 segments: scan launch
+    (40000, 2, 8, 16, torch.bfloat16, torch.int64, None, 8),       # short rows: 128 rows per workgroup
 ]
 
 
