@@ -1407,7 +1407,7 @@ extern "C" int ms_moe_token_permute_workspace_size(int64_t num_tokens, int64_t t
                "ms_moe_token_permute_workspace_size: num_experts_hint %lld exceeds %d", (long long)num_experts_hint,
                MS_MAX_EXPERTS);
     const SortPlan p = make_sort_plan(num_tokens * topk, num_experts_hint);
-    *bytes = static_cast<size_t>(p.nseg) * p.nbins * sizeof(int);
+    *bytes = p.small ? 0 : static_cast<size_t>(p.nseg) * p.nbins * sizeof(int);
     return MS_OK;
 }
 
@@ -1430,7 +1430,7 @@ extern "C" int ms_moe_token_permute(ms_stream_t stream_, const void *tokens, con
     MS_REQUIRE(tokens && indices && row_id_map && (permuted || num_out == 0), MS_ERR_INVALID_ARGUMENT,
                "ms_moe_token_permute: NULL tensor pointer");
     const SortPlan p = make_sort_plan(T * k, experts_hint);
-    const size_t need = static_cast<size_t>(p.nseg) * p.nbins * sizeof(int);
+    const size_t need = p.small ? 0 : static_cast<size_t>(p.nseg) * p.nbins * sizeof(int);
     MS_REQUIRE(workspace_bytes >= need && (need == 0 || workspace != nullptr), MS_ERR_WORKSPACE_TOO_SMALL,
                "ms_moe_token_permute: workspace %zu < %zu bytes", workspace_bytes, need);
     const int64_t row_bytes = H * dtype_size(dtype);
