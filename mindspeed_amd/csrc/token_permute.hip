@@ -849,8 +849,7 @@ __global__ __launch_bounds__(1024) void permute_fused_bins_kernel(
 //                    its own; the host picks this form while the table is small enough to read per workgroup.
 // To that it adds the keys of its segment in front of its first position, counted by all threads with LDS adds,
 // and its first wavefront runs the same stable scatter as sort_scatter_kernel over the workgroup's positions,
-// piece by piece where they cross a segment boundary.  The rows reach the copying threads through LDS; the
-// first vectors of the source rows are requested before the counting.
+// piece by piece where they cross a segment boundary.  The rows reach the copying threads through LDS.
 template <typename IdxT, typename VecT, bool SCANNED>
 __global__ __launch_bounds__(1024) void permute_scatter_rows_kernel(
     const VecT *__restrict__ tokens, VecT *__restrict__ permuted, const IdxT *__restrict__ idx, int n, int seg, int nseg,
@@ -882,10 +881,6 @@ __global__ __launch_bounds__(1024) void permute_scatter_rows_kernel(
     IdxT raw[KU];
 #pragma unroll
     for (int u = 0; u < KU; ++u) raw[u] = idx[min(seg_begin + u * nthreads + tid, n - 1)];
-    VecT v[8];   // first vectors of this thread's row: unconditional loads from clamped positions, in flight
-                 // while the keys above are counted
-#pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
     __syncthreads();
     for (int c = seg_begin; c < p0; c += KU * nthreads) {
         if (c != seg_begin) {
@@ -908,6 +903,14 @@ __global__ __launch_bounds__(1024) void permute_scatter_rows_kernel(
             atomicAdd(&first[e], c);                 // per-bin total for now
             if (sg < s0) atomicAdd(&pre[e], c);
         }
+    }
+    // The first vectors of this thread's row (clamped, unconditional loads), requested after the last load the
+    // counting needs - loads retire in order, so an earlier request would stall the counting until the rows are
+    // in - and in flight during the scan and the ranking below.
+    VecT v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+    if constexpr (!SCANNED) {
         __syncthreads();
         int carry = 0;
         for (int e0 = 0; e0 < nbins; e0 += nthreads) {
@@ -1152,6 +1155,127 @@ __global__ __launch_bounds__(1024) void routing_map_fused_kernel(
 #pragma unroll
             for (int u = 0; u < 8; ++u)
                 if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + c0 + u * lanes);
+        }
+    }
+}
+
+// Mask mode for any expert count (no drop-and-pad), two launches.  The map is cut into chunks of `chunk` tokens
+// (a power of two): routing_map_hist_kernel counts the set entries per (chunk, expert); every workgroup of
+// routing_map_ranked_kernel then owns a few tokens of one chunk, adds up the table (per expert: all chunks ->
+// first row of the expert after a scan over the experts; the chunks in front of its own), counts its chunk's
+// set entries in front of its first token, walks its own tokens in order, one thread per expert column, and
+// copies its tokens' rows, whose first vectors were requested before the counting.  Same outputs as the
+// sort-based path.
+__global__ __launch_bounds__(256) void routing_map_hist_kernel(const unsigned char *__restrict__ map, int num_tokens, int E,
+                                                               int chunk, int *__restrict__ hist) {
+    extern __shared__ int lds[];   // cnt[E]
+    const int tid = threadIdx.x;
+    for (int e = tid; e < E; e += 256) lds[e] = 0;
+    __syncthreads();
+    const int begin = blockIdx.x * chunk * E;
+    const int end = min(num_tokens, (static_cast<int>(blockIdx.x) + 1) * chunk) * E;
+    for (int i = begin + tid; i < end; i += 256)
+        if (map[i] != 0) atomicAdd(&lds[i % E], 1);
+    __syncthreads();
+    for (int e = tid; e < E; e += 256) hist[blockIdx.x * E + e] = lds[e];
+}
+
+template <typename VecT>
+__global__ __launch_bounds__(1024) void routing_map_ranked_kernel(
+    const VecT *__restrict__ tokens, VecT *__restrict__ permuted, const unsigned char *__restrict__ map, int num_tokens,
+    int E, int chunk, int nchunk, const int *__restrict__ hist, int num_rows, int32_t *__restrict__ row_id_map,
+    int32_t *__restrict__ sorted_flat, int64_t *__restrict__ tokens_per_expert, int vecs_per_row, int lanes,
+    int rows_per_block) {
+    // first[E], pre[E], cnt[E], scratch[32], ntok[rows_per_block], list[rows_per_block * E] (movers only),
+    // own[rows_per_block * E] bytes
+    extern __shared__ int lds[];
+    int *first = lds;
+    int *pre = first + E;
+    int *cnt = pre + E;
+    int *scratch = cnt + E;
+    int *ntok = scratch + 32;
+    int *list = ntok + rows_per_block;
+    unsigned char *own = reinterpret_cast<unsigned char *>(list + (tokens != nullptr ? rows_per_block * E : 0));
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    const int t0 = blockIdx.x * rows_per_block;
+    const int t1 = min(t0 + rows_per_block, num_tokens);
+    const int c0 = t0 / chunk;                  // rows_per_block divides chunk: all own tokens lie in chunk c0
+    const int split = t0 * E;                   // first own flat entry
+    const int own_n = (t1 - t0) * E;
+    const int local_row = tid / lanes;
+    const int lane = tid % lanes;
+    const int t = t0 + local_row;
+    const bool mover = tokens != nullptr && local_row < rows_per_block && t < num_tokens;
+    const VecT *src = tokens + static_cast<int64_t>(mover ? t : 0) * vecs_per_row;
+
+    for (int e = tid; e < 3 * E + 32 + rows_per_block; e += nthreads) lds[e] = 0;
+    for (int q = tid; q < own_n; q += nthreads) own[q] = map[split + q];
+    __syncthreads();
+    for (int i = c0 * chunk * E + tid; i < split; i += nthreads)       // this chunk's entries in front of the own ones
+        if (map[i] != 0) atomicAdd(&cnt[i % E], 1);
+    for (int i = tid; i < nchunk * E; i += nthreads) {
+        const int c = i / E;
+        const int count = hist[i];
+        atomicAdd(&first[i - c * E], count);    // per-expert total for now
+        if (c < c0) atomicAdd(&pre[i - c * E], count);
+    }
+    // The first vectors of this thread's row (clamped, unconditional loads), requested after the last load the
+    // ranking needs - loads retire in order, so an earlier request would stall the counting above until the rows
+    // are in - and in flight during the scan and the ranking below, which work out of LDS.
+    VecT v[8];
+    if (tokens != nullptr) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+    }
+    __syncthreads();
+    int carry = 0;
+    for (int e0 = 0; e0 < E; e0 += nthreads) {
+        const int e = e0 + tid;
+        const int total = e < E ? first[e] : 0;
+        const int start = carry + block_exclusive_scan(total, scratch);
+        if (e < E) {
+            first[e] = start;
+            if (blockIdx.x == 0 && tokens_per_expert != nullptr) tokens_per_expert[e] = total;
+        }
+        if (tid == nthreads - 1) scratch[16] = start + total;
+        __syncthreads();
+        carry = scratch[16];
+        __syncthreads();
+    }
+    if (blockIdx.x == 0)   // rows that nothing maps to (only if the caller's row count exceeds the set entries)
+        for (int r = carry + tid; r < num_rows; r += nthreads) sorted_flat[r] = -1;
+    for (int e = tid; e < E; e += nthreads) {
+        int next = first[e] + pre[e] + cnt[e];
+        for (int lt = 0; lt < t1 - t0; ++lt) {
+            const int q = lt * E + e;
+            int row = 0x7fffffff;               // unset or dropped: an id no row count reaches
+            if (own[q] != 0) {
+                if (next < num_rows) {
+                    row = next;
+                    sorted_flat[row] = split + q;
+                    if (tokens != nullptr) list[lt * E + atomicAdd(&ntok[lt], 1)] = row;
+                }
+                ++next;
+            }
+            row_id_map[split + q] = row;
+        }
+    }
+    __syncthreads();
+    if (!mover) return;
+    const int mine = ntok[local_row];
+    const int *d = list + local_row * E;
+    for (int cv = lane; cv < vecs_per_row; cv += 8 * lanes) {
+        if (cv != lane) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (cv + u * lanes < vecs_per_row) v[u] = src[cv + u * lanes];
+        }
+        for (int j = 0; j < mine; ++j) {
+            VecT *dst = permuted + static_cast<int64_t>(d[j]) * vecs_per_row;
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (cv + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + cv + u * lanes);
         }
     }
 }
@@ -1540,6 +1664,62 @@ RoutingPlan make_routing_plan(int64_t T, int64_t E, int pad) {
     r.total = r.sort_off + up(r.sort.small ? 0 : static_cast<size_t>(r.sort.nseg) * r.sort.nbins * sizeof(int));
     return r;
 }
+template <typename VecT>
+void launch_routing_map_ranked(hipStream_t stream, const void *tokens, void *permuted, const unsigned char *map, int64_t T,
+                               int64_t E, int chunk, int nchunk, const int *hist, int64_t num_rows, int32_t *row_id_map,
+                               int32_t *sorted_flat, int64_t *tpe, int64_t vecs, int lanes, int threads,
+                               int rows_per_block) {
+    const size_t ints = 3 * static_cast<size_t>(E) + 32 + rows_per_block +
+                        (tokens != nullptr ? static_cast<size_t>(rows_per_block) * E : 0);
+    const size_t lds = ints * sizeof(int) + ((static_cast<size_t>(rows_per_block) * E + 3) & ~static_cast<size_t>(3));
+    hipLaunchKernelGGL((ms::routing_map_ranked_kernel<VecT>), dim3(static_cast<unsigned>(ms::ceil_div(T, rows_per_block))),
+                       dim3(threads), lds, stream, static_cast<const VecT *>(tokens), static_cast<VecT *>(permuted), map,
+                       static_cast<int>(T), static_cast<int>(E), chunk, nchunk, hist, static_cast<int>(num_rows),
+                       row_id_map, sorted_flat, tpe, static_cast<int>(vecs), lanes, rows_per_block);
+}
+
+// Mask mode in two launches (chunk histogram, then ranking + row movement).  Returns -1 when the shape does not
+// fit (a workgroup's entries beyond what LDS holds, or chunks too large to count per workgroup): the caller
+// then takes the sort-based path.
+int routing_map_two_launches(hipStream_t stream, const void *tokens, const unsigned char *map, int64_t T, int64_t E,
+                             int64_t row_bytes, int dtype, int64_t num_rows, void *permuted, int32_t *row_id_map,
+                             int32_t *sorted_flat, int64_t *tpe, int *hist) {
+    using namespace ms;
+    int lanes = 1, threads = 1024, rows_per_block;
+    int64_t vecs = 1;
+    int vec_bytes = 16;
+    if (tokens != nullptr) {
+        if (!(row_bytes % 16 == 0 && aligned16(tokens) && aligned16(permuted))) vec_bytes = dtype == MS_FP32 ? 4 : 2;
+        vecs = row_bytes / vec_bytes;
+        lanes = row_layout(vecs).lanes;
+        while (threads > 256 && (ceil_div(T, threads / lanes) < 256 || (threads / lanes) * E > kFusedMaxLocal)) threads >>= 1;
+        rows_per_block = threads / lanes;
+        if (static_cast<int64_t>(rows_per_block) * E > kFusedMaxLocal) return -1;
+    } else {
+        rows_per_block = 1024;
+        while (rows_per_block > 1 && rows_per_block * E > 4 * kFusedMaxLocal) rows_per_block >>= 1;
+        threads = rows_per_block < 256 ? 256 : rows_per_block;
+    }
+    int chunk = rows_per_block;
+    while (ceil_div(T, chunk) * E > kScanInKernelMax) chunk <<= 1;
+    if (static_cast<int64_t>(chunk) * E > (1 << 16)) return -1;
+    const int nchunk = static_cast<int>(ceil_div(T, chunk));
+    hipLaunchKernelGGL(routing_map_hist_kernel, dim3(nchunk), dim3(256), static_cast<size_t>(E) * sizeof(int), stream, map,
+                       static_cast<int>(T), static_cast<int>(E), chunk, hist);
+    MS_CHECK_LAUNCH("routing_map_hist_kernel");
+    if (vec_bytes == 16)
+        launch_routing_map_ranked<v16>(stream, tokens, permuted, map, T, E, chunk, nchunk, hist, num_rows, row_id_map,
+                                       sorted_flat, tpe, vecs, lanes, threads, rows_per_block);
+    else if (vec_bytes == 4)
+        launch_routing_map_ranked<uint32_t>(stream, tokens, permuted, map, T, E, chunk, nchunk, hist, num_rows, row_id_map,
+                                            sorted_flat, tpe, vecs, lanes, threads, rows_per_block);
+    else
+        launch_routing_map_ranked<uint16_t>(stream, tokens, permuted, map, T, E, chunk, nchunk, hist, num_rows, row_id_map,
+                                            sorted_flat, tpe, vecs, lanes, threads, rows_per_block);
+    MS_CHECK_LAUNCH("routing_map_ranked_kernel");
+    return MS_OK;
+}
+
 int check_routing(const char *fn, int64_t T, int64_t E, int pad) {
     MS_REQUIRE(T >= 0 && E >= 1, MS_ERR_INVALID_ARGUMENT, "%s: need num_tokens >= 0, num_experts >= 1", fn);
     MS_REQUIRE((pad ? 2 * E : E + 1) <= MS_MAX_EXPERTS, MS_ERR_UNSUPPORTED, "%s: num_experts %lld too large (limit %d%s)",
@@ -1602,6 +1782,12 @@ extern "C" int ms_moe_routing_map_permute(ms_stream_t stream_, const void *token
                fn, workspace_bytes, r.total);
     MS_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7u) == 0, MS_ERR_INVALID_ARGUMENT, "%s: workspace must be 8-byte aligned", fn);
     char *ws = static_cast<char *>(workspace);
+    if (!drop_and_pad) {
+        const int rc = routing_map_two_launches(stream, tokens, static_cast<const unsigned char *>(routing_map), T, E,
+                                                row_bytes_f, dtype, num_rows, permuted, row_id_map, sorted_flat,
+                                                tokens_per_expert, reinterpret_cast<int *>(ws + r.keys_off));
+        if (rc != -1) return rc;
+    }
     int32_t *keys = reinterpret_cast<int32_t *>(ws + r.keys_off);
     int64_t *counts = reinterpret_cast<int64_t *>(ws + r.counts_off);
     const int n = static_cast<int>(r.n);
