@@ -388,35 +388,81 @@ __global__ __launch_bounds__(256) void permute_rows_kernel(const VecT *__restric
     }
 }
 
+// The slots of token t whose row id lies in [0, num_rows), in slot order, into an LDS list (row id, weight and,
+// if asked for, slot number); returns their count.  For the routing-map form, where a token has one slot per
+// expert and only a few are set: the row loops then run over the list instead of over all slots.  The `lanes`
+// threads of a token (a power of two, part of one wavefront) look at `lanes` slots at a time and place the
+// valid ones with a ballot.  Probability gradients of the other slots are zeroed here when `zero` is given.
+constexpr int kCompactMaxLocal = 2048;   // (token, slot) pairs of one workgroup that the lists hold
+template <typename DT>
+__device__ __forceinline__ int compact_slots(const int32_t *__restrict__ row_id_map,
+                                             const typename DT::storage *__restrict__ probs, int t, int topk,
+                                             int num_rows, int lane, int lanes, int *ld, float *lw, int *lj,
+                                             typename DT::storage *__restrict__ zero) {
+    const int wl = threadIdx.x & 63;
+    const int group0 = wl - lane;
+    const unsigned long long group = (lanes == 64 ? ~0ull : ((1ull << lanes) - 1ull)) << group0;
+    const unsigned long long below = (1ull << wl) - 1ull;
+    int count = 0;
+    for (int j0 = 0; j0 < topk; j0 += lanes) {
+        const int j = j0 + lane;
+        const int64_t flat = static_cast<int64_t>(t) * topk + j;
+        const int d = j < topk ? row_id_map[flat] : num_rows;
+        const bool valid = j < topk && static_cast<unsigned>(d) < static_cast<unsigned>(num_rows);
+        const unsigned long long bal = __ballot(valid) & group;
+        if (valid) {
+            const int pos = count + __popcll(bal & below);
+            ld[pos] = d;
+            lw[pos] = probs != nullptr ? DT::to_float(probs[flat]) : 1.f;
+            if (lj != nullptr) lj[pos] = j;
+        } else if (zero != nullptr && j < topk) {
+            zero[flat] = DT::from_float(0.f);
+        }
+        count += __popcll(bal);
+    }
+    __builtin_amdgcn_wave_barrier();   // the list is read by the same lanes' wavefront only
+    return count;
+}
+
 // out[t] = sum_j w[t,j] * rows[row_id_map[t*k+j]] ; w == nullptr -> unweighted.
 // VEC: elements per thread access (16 bytes worth, or 1 for the unaligned path).
 // Row ids and weights are read once per thread; per group of U output vectors the row loads of up to JB
 // slots are independent and issued together; accumulation is fp32 in registers, slot by slot, one rounding.
-template <typename DT, int VEC, int JB, int U>
+template <typename DT, int VEC, int JB, int U, bool COMPACT>
 __global__ __launch_bounds__(256) void gather_combine_kernel(
     const typename DT::storage *__restrict__ rows, const int32_t *__restrict__ row_id_map,
     const typename DT::storage *__restrict__ probs, typename DT::storage *__restrict__ out,
     int num_tokens, int topk, int hidden, int num_rows, int lanes) {
     using S = typename DT::storage;
+    extern __shared__ int lds[];   // COMPACT: row ids [rows_per_block][topk], then weights
     const int local_row = threadIdx.x / lanes;
     const int lane = threadIdx.x % lanes;
     const int t = blockIdx.x * (256 / lanes) + local_row;
     if (t >= num_tokens) return;
     const int vecs = hidden / VEC;
+    int *ld = lds + local_row * topk;
+    float *lw = reinterpret_cast<float *>(lds + (256 / lanes) * topk) + local_row * topk;
+    int nslots = topk;
+    if constexpr (COMPACT) nslots = compact_slots<DT>(row_id_map, probs, t, topk, num_rows, lane, lanes, ld, lw, nullptr, nullptr);
     for (int c0 = lane; c0 < vecs; c0 += U * lanes) {
         float acc[U][VEC];
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int e = 0; e < VEC; ++e) acc[u][e] = 0.f;
-        for (int j0 = 0; j0 < topk; j0 += JB) {
+        for (int j0 = 0; j0 < nslots; j0 += JB) {
             int d[JB];
             float w[JB];
 #pragma unroll
             for (int j = 0; j < JB; ++j) {
-                const int64_t flat = static_cast<int64_t>(t) * topk + j0 + j;
-                d[j] = j0 + j < topk ? row_id_map[flat] : num_rows;
-                w[j] = (probs != nullptr && j0 + j < topk) ? DT::to_float(probs[flat]) : 1.f;
+                if constexpr (COMPACT) {
+                    d[j] = j0 + j < nslots ? ld[j0 + j] : num_rows;
+                    w[j] = j0 + j < nslots ? lw[j0 + j] : 1.f;
+                } else {
+                    const int64_t flat = static_cast<int64_t>(t) * topk + j0 + j;
+                    d[j] = j0 + j < topk ? row_id_map[flat] : num_rows;
+                    w[j] = (probs != nullptr && j0 + j < topk) ? DT::to_float(probs[flat]) : 1.f;
+                }
             }
             S tmp[JB][U][VEC];
 #pragma unroll
@@ -468,7 +514,7 @@ __global__ __launch_bounds__(256) void gather_combine_kernel(
 // `lanes` threads (a power of two, one wavefront at most) share a token, so the dot products are folded with
 // lane shuffles and the kernel has no barrier.  Per chunk of U vectors a thread reads dY once and has the
 // loads of up to JB slots' rows in flight together.
-template <typename DT, int VEC, int JB, int U>
+template <typename DT, int VEC, int JB, int U, bool COMPACT>
 __global__ __launch_bounds__(256) void unpermute_grad_kernel(
     const typename DT::storage *__restrict__ permuted, const typename DT::storage *__restrict__ grad_out,
     const int32_t *__restrict__ row_id_map, const typename DT::storage *__restrict__ probs,
@@ -482,14 +528,26 @@ __global__ __launch_bounds__(256) void unpermute_grad_kernel(
     const int vecs = hidden / VEC;
     const S *gy = grad_out + static_cast<int64_t>(t) * hidden;
     const bool want_dot = grad_probs != nullptr;
-    for (int j0 = 0; j0 < topk; j0 += JB) {
+    extern __shared__ int lds[];   // COMPACT: row ids [rows_per_block][topk], weights, slot numbers
+    int *ld = lds + local_row * topk;
+    float *lw = reinterpret_cast<float *>(lds + (256 / lanes) * topk) + local_row * topk;
+    int *lj = lds + 2 * (256 / lanes) * topk + local_row * topk;
+    int nslots = topk;
+    if constexpr (COMPACT)
+        nslots = compact_slots<DT>(row_id_map, probs, t, topk, num_rows, lane, lanes, ld, lw, lj, grad_probs);
+    for (int j0 = 0; j0 < nslots; j0 += JB) {
         int d[JB];
         float w[JB], dot[JB];
 #pragma unroll
         for (int j = 0; j < JB; ++j) {
-            const int64_t flat = static_cast<int64_t>(t) * topk + j0 + j;
-            d[j] = j0 + j < topk ? row_id_map[flat] : num_rows;          // ids outside [0, num_rows): dropped
-            w[j] = (probs != nullptr && j0 + j < topk) ? DT::to_float(probs[flat]) : 1.f;
+            if constexpr (COMPACT) {
+                d[j] = j0 + j < nslots ? ld[j0 + j] : num_rows;
+                w[j] = j0 + j < nslots ? lw[j0 + j] : 1.f;
+            } else {
+                const int64_t flat = static_cast<int64_t>(t) * topk + j0 + j;
+                d[j] = j0 + j < topk ? row_id_map[flat] : num_rows;          // ids outside [0, num_rows): dropped
+                w[j] = (probs != nullptr && j0 + j < topk) ? DT::to_float(probs[flat]) : 1.f;
+            }
             dot[j] = 0.f;
         }
         for (int c0 = lane; c0 < vecs; c0 += U * lanes) {
@@ -553,7 +611,10 @@ __global__ __launch_bounds__(256) void unpermute_grad_kernel(
             for (int j = 0; j < JB; ++j) {
                 float s = dot[j];
                 for (int dlt = lanes >> 1; dlt > 0; dlt >>= 1) s += __shfl_xor(s, dlt, 64);
-                if (lane == 0 && j0 + j < topk) grad_probs[static_cast<int64_t>(t) * topk + j0 + j] = DT::from_float(s);
+                if (lane == 0 && j0 + j < nslots) {
+                    const int slot = COMPACT ? lj[j0 + j] : j0 + j;
+                    grad_probs[static_cast<int64_t>(t) * topk + slot] = DT::from_float(s);
+                }
             }
         }
     }
@@ -1468,12 +1529,19 @@ int launch_gather_combine(hipStream_t stream, const void *rows, const int32_t *m
 #define MS_GC_ARGS                                                                                                  \
     static_cast<const S *>(rows), map, static_cast<const S *>(probs), static_cast<S *>(out), static_cast<int>(T),   \
         static_cast<int>(k), static_cast<int>(H), static_cast<int>(num_rows), rl.lanes
-    if (!vec_ok) {
-        hipLaunchKernelGGL((gather_combine_kernel<DT, 1, 8, 2>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
+    // many slots per token (the routing-map form has one per expert): list the valid ones first
+    const bool compact = k > 8 && rl.rows_per_block * k <= kCompactMaxLocal;
+    const size_t lds = compact ? static_cast<size_t>(2) * rl.rows_per_block * k * sizeof(int) : 0;
+    if (!vec_ok && compact) {
+        hipLaunchKernelGGL((gather_combine_kernel<DT, 1, 8, 2, true>), dim3(blocks), dim3(256), lds, stream, MS_GC_ARGS);
+    } else if (!vec_ok) {
+        hipLaunchKernelGGL((gather_combine_kernel<DT, 1, 8, 2, false>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
+    } else if (compact) {
+        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC, 8, 2, true>), dim3(blocks), dim3(256), lds, stream, MS_GC_ARGS);
     } else if (k <= 2) {
-        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC, 2, 4>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
+        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC, 2, 4, false>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
     } else {
-        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC, 8, 2>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
+        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC, 8, 2, false>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
     }
 #undef MS_GC_ARGS
     MS_CHECK_LAUNCH("gather_combine_kernel");
@@ -1494,12 +1562,18 @@ int launch_unpermute_grad(hipStream_t stream, const void *permuted, const void *
     static_cast<const S *>(permuted), static_cast<const S *>(gy), map, static_cast<const S *>(probs),                \
         static_cast<S *>(gperm), static_cast<S *>(gprobs), static_cast<int>(T), static_cast<int>(k),                 \
         static_cast<int>(H), static_cast<int>(num_rows), rl.lanes
-    if (!vec_ok) {
-        hipLaunchKernelGGL((unpermute_grad_kernel<DT, 1, 4, 4>), grid, dim3(256), 0, stream, MS_UG_ARGS);
+    const bool compact = k > 8 && rl.rows_per_block * k <= kCompactMaxLocal;
+    const size_t lds = compact ? static_cast<size_t>(3) * rl.rows_per_block * k * sizeof(int) : 0;
+    if (!vec_ok && compact) {
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, 1, 4, 4, true>), grid, dim3(256), lds, stream, MS_UG_ARGS);
+    } else if (!vec_ok) {
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, 1, 4, 4, false>), grid, dim3(256), 0, stream, MS_UG_ARGS);
+    } else if (compact) {
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC, 4, 2, true>), grid, dim3(256), lds, stream, MS_UG_ARGS);
     } else if (k <= 2) {
-        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC, 2, 4>), grid, dim3(256), 0, stream, MS_UG_ARGS);
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC, 2, 4, false>), grid, dim3(256), 0, stream, MS_UG_ARGS);
     } else {
-        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC, 4, 2>), grid, dim3(256), 0, stream, MS_UG_ARGS);
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC, 4, 2, false>), grid, dim3(256), 0, stream, MS_UG_ARGS);
     }
 #undef MS_UG_ARGS
     MS_CHECK_LAUNCH("unpermute_grad_kernel");

@@ -14,6 +14,8 @@ over that average, next to the 8 TB/s HBM peak.  The ops:
     unpermute       ms_moe_token_unpermute        probability-weighted top-k gather
     unpermute_grad  ms_moe_token_unpermute_grad   grad of rows and of probabilities
     permute_grad    ms_moe_token_permute_grad     unweighted top-k gather
+    unpermute_mask, unpermute_mask_grad, permute_mask_grad
+                    the three gathers above driven by the routing-map form's row map (top-k = experts)
     copy            ms_copy_bytes                 plain copy of the permuted rows, for orientation
 """
 from __future__ import annotations
@@ -56,6 +58,8 @@ def measure(num_tokens=4096, hidden=4096, num_experts=8, topk=2, dtype=torch.bfl
     gperm = torch.empty_like(perm)
     gprobs = torch.empty_like(probs)
     copy_dst = torch.empty_like(perm)
+    probs_mask = torch.zeros(T, E, dtype=dtype, device=dev).scatter_(1, idx, probs)
+    gprobs_mask = torch.empty_like(probs_mask)
     nbytes = ctypes.c_size_t(0)
     _lib.check(lib.ms_moe_token_permute_workspace_size(T, K, E, ctypes.byref(nbytes)), "workspace_size")
     ws = _lib.workspace(nbytes.value, dev)
@@ -79,6 +83,17 @@ def measure(num_tokens=4096, hidden=4096, num_experts=8, topk=2, dtype=torch.bfl
             flop_counter.unpermute_grad_bytes(T, K, H, elem)),
         "permute_grad": (lambda: lib.ms_moe_token_permute_grad(
             stream, P(perm), P(row_id_map), T, K, H, code, rows, P(out)), flop_counter.permute_grad_bytes(T, K, H, elem)),
+        # the routing-map form of the three gathers: the same entry points with top-k = experts, a [tokens, experts]
+        # row map whose unset entries hold an id past the last row, and [tokens, experts] probabilities
+        "unpermute_mask": (lambda: lib.ms_moe_token_unpermute(
+            stream, P(perm), P(mask_map), P(probs_mask), T, E, H, code, rows, P(out)),
+            flop_counter.unpermute_bytes(T, K, H, elem) + T * (E - K) * (4 + elem)),
+        "unpermute_mask_grad": (lambda: lib.ms_moe_token_unpermute_grad(
+            stream, P(perm), P(gy), P(mask_map), P(probs_mask), T, E, H, code, rows, P(gperm), P(gprobs_mask)),
+            flop_counter.unpermute_grad_bytes(T, K, H, elem) + T * (E - K) * (4 + 2 * elem)),
+        "permute_mask_grad": (lambda: lib.ms_moe_token_permute_grad(
+            stream, P(perm), P(mask_map), T, E, H, code, rows, P(out)),
+            flop_counter.permute_grad_bytes(T, K, H, elem) + T * (E - K) * 4),
         "copy": (lambda: lib.ms_copy_bytes(stream, P(perm), P(copy_dst), perm.numel() * elem), 2 * perm.numel() * elem),
     }
     result = {}
@@ -111,7 +126,7 @@ def main():
     res = measure(a.tokens, a.hidden, a.experts, a.topk, torch.bfloat16, a.iters, a.warmup)
     print(f"{a.tokens} tokens x hidden {a.hidden}, {a.experts} experts, top-{a.topk}, bf16; {a.iters} launches per op")
     for name, r in res.items():
-        print(f"{name:15s} {r['avg_us']:8.2f} us  {r['gbs']:8.1f} GB/s  {r['frac_of_hbm_peak']:.3f} of 8 TB/s  "
+        print(f"{name:19s} {r['avg_us']:8.2f} us  {r['gbs']:8.1f} GB/s  {r['frac_of_hbm_peak']:.3f} of 8 TB/s  "
               f"({r['bytes_per_launch'] / 1e6:.1f} MB per launch)", flush=True)
 
 
