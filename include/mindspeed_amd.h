@@ -46,8 +46,10 @@ typedef enum ms_status {
 typedef enum ms_dtype { MS_BF16 = 0, MS_FP16 = 1, MS_FP32 = 2 } ms_dtype;
 typedef enum ms_index_dtype { MS_INT32 = 0, MS_INT64 = 1 } ms_index_dtype;
 
-/* Largest expert id + 1 the permute sort accepts.  Ids outside [0, limit) are
- * clamped into range for memory safety; results are then unspecified. */
+/* Largest expert id + 1 the permute sort accepts.  The sort's key range is the
+ * power of two that holds num_experts_hint (MS_MAX_EXPERTS without a hint); ids
+ * outside it are clamped into it (negative ones to 0, large ones to the last key)
+ * and sorted as such, so no id can address memory out of range. */
 #define MS_MAX_EXPERTS 1024
 
 /* Library identification and error text (thread-local, never NULL). */
