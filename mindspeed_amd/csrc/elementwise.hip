@@ -106,36 +106,121 @@ __global__ __launch_bounds__(256) void swiglu_grad_kernel(const typename DT::sto
     }
 }
 
-// row_map[r] = source row of output row r for out = cat(chunks[sorted_idxs[i]]).
-// One block; num_chunks is small (experts x ranks).
-__global__ __launch_bounds__(256) void chunk_row_map_kernel(const int64_t *__restrict__ split_sizes,
-                                                            const int64_t *__restrict__ sorted_idxs,
-                                                            int num_chunks, int rows, int32_t *row_map) {
-    extern __shared__ int64_t sh[];  // src_start[num_chunks], dst_start[num_chunks]
-    int64_t *src_start = sh;
-    int64_t *dst_start = sh + num_chunks;
-    if (threadIdx.x == 0) {
-        int64_t acc = 0;
-        for (int i = 0; i < num_chunks; ++i) { src_start[i] = acc; acc += split_sizes[i]; }
-        acc = 0;
-        for (int i = 0; i < num_chunks; ++i) {
-            const int64_t src = sorted_idxs[i];
-            dst_start[i] = acc;
-            if (src >= 0 && src < num_chunks) acc += split_sizes[src];
+// Exclusive scan of one int per thread over a block of up to 1024 threads (scratch: 16 ints).
+__device__ __forceinline__ int block_exclusive_scan(int v, int *scratch) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    int incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+    }
+    if (lane == 63) scratch[wave] = incl;
+    __syncthreads();
+    if (wave == 0) {
+        const int nw = (blockDim.x + 63) >> 6;
+        int w = lane < nw ? scratch[lane] : 0;
+        int wi = w;
+#pragma unroll
+        for (int d = 1; d < 16; d <<= 1) {
+            const int up = __shfl_up(wi, d, 64);
+            if (lane >= d) wi += up;
         }
+        if (lane < nw) scratch[lane] = wi - w;
     }
     __syncthreads();
-    for (int i = 0; i < num_chunks; ++i) {
-        const int64_t src = sorted_idxs[i];
-        if (src < 0 || src >= num_chunks) continue;  // malformed index: skip rather than read out of bounds
-        const int64_t len = split_sizes[src];
-        for (int64_t r = threadIdx.x; r < len; r += blockDim.x) {
-            const int64_t o = dst_start[i] + r;
-            if (o < rows) row_map[o] = static_cast<int32_t>(src_start[src] + r);
+    return incl - v + scratch[wave];
+}
+
+// out = cat(chunks[sorted_idxs[i]] for i) in one launch: row_map[r] = source row of output row r, the rows
+// themselves, and optionally one probability per row.  Every workgroup scans the chunk sizes itself (in input
+// order -> first source row of every chunk; in output order -> first output row of every position; num_chunks is
+// experts x ranks, a few thousand at most), finds the position of each of its output rows by bisection, and
+// copies the rows with `lanes` threads per row, eight 16-byte loads in flight per thread.  Output rows past the
+// sum of the sizes get row_map = -1 and are left alone; malformed chunk indices count as empty chunks.
+template <typename VecT>
+__global__ __launch_bounds__(1024) void sort_chunks_kernel(
+    const VecT *__restrict__ in, VecT *__restrict__ out, const int64_t *__restrict__ split_sizes,
+    const int64_t *__restrict__ sorted_idxs, int num_chunks, int rows, int vecs_per_row, int lanes,
+    const void *__restrict__ probs, void *__restrict__ out_probs, int probs_bytes, int32_t *__restrict__ row_map) {
+    extern __shared__ int lds[];   // src_start[num_chunks], dst_start[num_chunks + 1], src_of[num_chunks], scratch[32]
+    int *src_start = lds;
+    int *dst_start = lds + num_chunks;
+    int *src_of = dst_start + num_chunks + 1;
+    int *scratch = src_of + num_chunks;
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    int carry_s = 0, carry_d = 0;
+    for (int c0 = 0; c0 < num_chunks; c0 += nthreads) {
+        const int i = c0 + tid;
+        int size = 0, moved = 0, src = -1;
+        if (i < num_chunks) {
+            const int64_t sz = split_sizes[i];
+            size = static_cast<int>(sz < 0 ? 0 : (sz > rows ? rows : sz));
+            const int64_t sidx = sorted_idxs[i];
+            if (sidx >= 0 && sidx < num_chunks) {
+                src = static_cast<int>(sidx);
+                const int64_t ms = split_sizes[src];
+                moved = static_cast<int>(ms < 0 ? 0 : (ms > rows ? rows : ms));
+            }
         }
+        const int s_ex = carry_s + block_exclusive_scan(size, scratch);
+        const int d_ex = carry_d + block_exclusive_scan(moved, scratch);
+        if (i < num_chunks) {
+            src_start[i] = s_ex;
+            dst_start[i] = d_ex;
+            src_of[i] = src;
+        }
+        if (tid == nthreads - 1) {
+            scratch[16] = s_ex + size;
+            scratch[17] = d_ex + moved;
+        }
+        __syncthreads();
+        carry_s = scratch[16];
+        carry_d = scratch[17];
+        __syncthreads();
+    }
+    if (tid == 0) dst_start[num_chunks] = carry_d;
+    __syncthreads();
+
+    const int local_row = tid / lanes;
+    const int lane = tid % lanes;
+    const int r = blockIdx.x * (nthreads / lanes) + local_row;
+    if (r >= rows) return;
+    int lo = 0, hi = num_chunks + 1;            // last position with dst_start <= r
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (dst_start[mid] <= r) lo = mid; else hi = mid;
+    }
+    int m = -1;
+    if (lo < num_chunks && r < dst_start[num_chunks] && src_of[lo] >= 0) {
+        m = src_start[src_of[lo]] + (r - dst_start[lo]);
+        if (static_cast<unsigned>(m) >= static_cast<unsigned>(rows)) m = -1;   // sizes that run past the input
+    }
+    if (lane == 0) {
+        row_map[r] = m;
+        if (probs != nullptr && m >= 0) {
+            if (probs_bytes == 4) static_cast<uint32_t *>(out_probs)[r] = static_cast<const uint32_t *>(probs)[m];
+            else static_cast<uint16_t *>(out_probs)[r] = static_cast<const uint16_t *>(probs)[m];
+        }
+    }
+    if (m < 0) return;
+    const VecT *src_row = in + static_cast<int64_t>(m) * vecs_per_row;
+    VecT *dst_row = out + static_cast<int64_t>(r) * vecs_per_row;
+    for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
+        VecT v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (c0 + u * lanes < vecs_per_row) v[u] = MS_NT_LOAD(src_row + c0 + u * lanes);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst_row + c0 + u * lanes);
     }
 }
 
+// out[r] = in[row_map[r]] (inverse: out[row_map[r]] = in[r]); `lanes` threads per row, eight 16-byte loads in
+// flight per thread.  Map entries outside [0, rows) move nothing.
 template <typename VecT>
 __global__ __launch_bounds__(256) void gather_rows_kernel(const VecT *__restrict__ in, VecT *__restrict__ out,
                                                           const int32_t *__restrict__ row_map, int rows,
@@ -145,19 +230,31 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const VecT *__restrict
     const int r = blockIdx.x * (256 / lanes) + local_row;
     if (r >= rows) return;
     const int m = row_map[r];
-    if (static_cast<unsigned>(m) >= static_cast<unsigned>(rows)) return;   // corrupt map entry: touch nothing
-    const int64_t s = inverse ? r : m;
-    const int64_t d = inverse ? m : r;
-    for (int c = lane; c < vecs_per_row; c += lanes)
-        MS_NT_STORE(MS_NT_LOAD(in + s * vecs_per_row + c), out + d * vecs_per_row + c);
+    if (static_cast<unsigned>(m) >= static_cast<unsigned>(rows)) return;
+    const VecT *src_row = in + static_cast<int64_t>(inverse ? r : m) * vecs_per_row;
+    VecT *dst_row = out + static_cast<int64_t>(inverse ? m : r) * vecs_per_row;
+    for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
+        VecT v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (c0 + u * lanes < vecs_per_row) v[u] = MS_NT_LOAD(src_row + c0 + u * lanes);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst_row + c0 + u * lanes);
+    }
+}
+
+inline int row_lanes(int64_t vecs) {
+    int lanes = 1;
+    while (lanes < 64 && lanes < vecs) lanes <<= 1;   // one wavefront per row at most
+    return lanes;
 }
 
 template <typename VecT>
 int launch_gather_rows(hipStream_t stream, const void *in, void *out, const int32_t *map, int64_t rows,
                        int64_t row_bytes, int inverse) {
     const int64_t vecs = row_bytes / sizeof(VecT);
-    int lanes = 1;
-    while (lanes < 256 && lanes < vecs) lanes <<= 1;
+    const int lanes = row_lanes(vecs);
     const int64_t blocks = ceil_div(rows, 256 / lanes);
     hipLaunchKernelGGL(gather_rows_kernel<VecT>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
                        static_cast<const VecT *>(in), static_cast<VecT *>(out), map, static_cast<int>(rows),
@@ -173,6 +270,24 @@ int gather_rows_any(hipStream_t stream, const void *in, void *out, const int32_t
         return launch_gather_rows<v16>(stream, in, out, map, rows, row_bytes, inverse);
     if (dtype == MS_FP32) return launch_gather_rows<uint32_t>(stream, in, out, map, rows, row_bytes, inverse);
     return launch_gather_rows<uint16_t>(stream, in, out, map, rows, row_bytes, inverse);
+}
+
+template <typename VecT>
+int launch_sort_chunks(hipStream_t stream, const void *in, void *out, const int64_t *split_sizes,
+                       const int64_t *sorted_idxs, int64_t num_chunks, int64_t rows, int64_t row_bytes, const void *probs,
+                       void *out_probs, int probs_bytes, int32_t *row_map) {
+    const int64_t vecs = row_bytes / sizeof(VecT);
+    const int lanes = row_lanes(vecs);
+    // fat workgroups repeat the scan of the chunk sizes less often; keep one per compute unit
+    int threads = 1024;
+    while (threads > 256 && ceil_div(rows, threads / lanes) < 256) threads >>= 1;
+    const size_t lds = (3 * static_cast<size_t>(num_chunks) + 1 + 32) * sizeof(int);
+    hipLaunchKernelGGL(sort_chunks_kernel<VecT>, dim3(static_cast<unsigned>(ceil_div(rows, threads / lanes))), dim3(threads),
+                       lds, stream, static_cast<const VecT *>(in), static_cast<VecT *>(out), split_sizes, sorted_idxs,
+                       static_cast<int>(num_chunks), static_cast<int>(rows), static_cast<int>(vecs), lanes, probs,
+                       out_probs, probs_bytes, row_map);
+    MS_CHECK_LAUNCH("sort_chunks_kernel");
+    return MS_OK;
 }
 
 template <typename DT>
@@ -279,13 +394,19 @@ extern "C" int ms_sort_chunks(ms_stream_t stream_, const void *input, const int6
     MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED, "ms_sort_chunks: bad dtype");
     MS_REQUIRE((probs == nullptr) == (out_probs == nullptr), MS_ERR_INVALID_ARGUMENT,
                "ms_sort_chunks: probs and out_probs must be given together");
+    MS_REQUIRE(probs == nullptr || probs_dtype == MS_BF16 || probs_dtype == MS_FP16 || probs_dtype == MS_FP32,
+               MS_ERR_UNSUPPORTED, "ms_sort_chunks: bad probs dtype");
     if (rows == 0) return MS_OK;
     MS_REQUIRE(input && split_sizes && sorted_idxs && out && row_map, MS_ERR_INVALID_ARGUMENT,
                "ms_sort_chunks: NULL tensor pointer");
-    hipLaunchKernelGGL(chunk_row_map_kernel, dim3(1), dim3(256), 2 * num_chunks * sizeof(int64_t), stream, split_sizes,
-                       sorted_idxs, static_cast<int>(num_chunks), static_cast<int>(rows), row_map);
-    MS_CHECK_LAUNCH("chunk_row_map_kernel");
-    if (int rc = gather_rows_any(stream, input, out, row_map, rows, hidden, dtype, 0)) return rc;
-    if (probs != nullptr) return gather_rows_any(stream, probs, out_probs, row_map, rows, 1, probs_dtype, 0);
-    return MS_OK;
+    const int64_t row_bytes = hidden * dtype_size(dtype);
+    const int probs_bytes = probs != nullptr ? static_cast<int>(dtype_size(probs_dtype)) : 0;
+    if (row_bytes % 16 == 0 && aligned16(input) && aligned16(out))
+        return launch_sort_chunks<v16>(stream, input, out, split_sizes, sorted_idxs, num_chunks, rows, row_bytes, probs,
+                                       out_probs, probs_bytes, row_map);
+    if (dtype == MS_FP32)
+        return launch_sort_chunks<uint32_t>(stream, input, out, split_sizes, sorted_idxs, num_chunks, rows, row_bytes, probs,
+                                            out_probs, probs_bytes, row_map);
+    return launch_sort_chunks<uint16_t>(stream, input, out, split_sizes, sorted_idxs, num_chunks, rows, row_bytes, probs,
+                                        out_probs, probs_bytes, row_map);
 }

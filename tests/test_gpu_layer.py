@@ -70,6 +70,37 @@ def test_sort_chunks(nchunks, rows, hidden, device):
     assert none is None and torch.equal(out2.cpu(), eo)
 
 
+@pytest.mark.parametrize("dtype,pdt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float32),
+                                       (torch.float32, torch.float32)])
+@pytest.mark.parametrize("nchunks,rows,hidden", [(64, 8192, 512), (1500, 6000, 24), (2600, 40000, 8), (7, 300, 13)])
+def test_sort_chunks_sizes_and_dtypes(nchunks, rows, hidden, dtype, pdt, device):
+    """Many chunks (more than one scan pass), empty chunks, every dtype and the element path; a pure row copy,
+    so every output is exact.  Chunk counts follow experts x ranks of the reference's dispatcher
+    (mindspeed/core/transformer/moe/moe_feature/overlap/moe_common.py:377-398)."""
+    say("sort_chunks case", nchunks, rows, hidden, dtype, pdt)
+    gen = torch.Generator().manual_seed(nchunks + rows)
+    cuts = torch.sort(torch.randint(0, rows + 1, (nchunks - 1,), generator=gen))[0]
+    cuts[: nchunks // 4] = cuts[nchunks // 4]                 # a run of empty chunks at the front
+    sizes = torch.diff(torch.cat([torch.tensor([0]), cuts, torch.tensor([rows])]))
+    order = torch.randperm(nchunks, generator=gen)
+    x = torch.randn(rows, hidden, generator=gen).to(dtype)
+    p = torch.rand(rows, generator=gen).to(pdt)
+    eo, ep = O.sort_chunks_by_idxs(x, sizes, order, p)
+    xd = x.to(device).requires_grad_(True)
+    pd = p.to(device).requires_grad_(True)
+    out, outp = ops.sort_chunks_by_idxs(xd, sizes.to(device), order.to(device), pd)
+    assert torch.equal(out.cpu(), eo) and torch.equal(outp.cpu(), ep)
+    g = torch.randn(rows, hidden, generator=gen).to(dtype)
+    gp = torch.rand(rows, generator=gen).to(pdt)
+    torch.autograd.backward((out, outp), (g.to(device), gp.to(device)))
+    starts = torch.cat([torch.tensor([0]), torch.cumsum(sizes, 0)])
+    src_rows = torch.cat([torch.arange(starts[i], starts[i] + sizes[i]) for i in order.tolist()])
+    exp_g, exp_gp = torch.empty_like(g), torch.empty_like(gp)
+    exp_g[src_rows] = g
+    exp_gp[src_rows] = gp
+    assert torch.equal(xd.grad.cpu(), exp_g) and torch.equal(pd.grad.cpu(), exp_gp)
+
+
 def test_layer_fp64_fixture(device):
     g = np.load(os.path.join(GOLDEN, "layer_fp64.npz"))
     x, idx, p = (torch.from_numpy(g[k]).to(device) for k in ("x", "idx", "p"))
