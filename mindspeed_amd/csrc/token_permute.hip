@@ -1358,7 +1358,12 @@ inline SortPlan make_sort_plan(int64_t n, int64_t experts_hint) {
         p.nbits++;
     }
     p.small = n <= kSmallSortMax;
+    // 1024 positions per segment; beyond 128 segments the segments grow (up to 4096 positions) before their number
+    // does: the scan over the segments is a serial loop per bin, while a scatter workgroup counts at most one
+    // segment's keys in front of its own positions
     int64_t seg = 1024;
+    if (ceil_div(n, seg) > 128) seg = (ceil_div(n, 128) + 63) / 64 * 64;
+    if (seg > 4096) seg = 4096;
     if (ceil_div(n, seg) > kMaxSegments) seg = (ceil_div(n, kMaxSegments) + 63) / 64 * 64;
     p.seg = static_cast<int>(seg);
     p.nseg = static_cast<int>(ceil_div(n, seg));
