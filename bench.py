@@ -31,7 +31,7 @@ MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}   # dense, published
 # HBM bytes per launch of the dominant kernel (forward grouped matmul, fc1/fc2 average) from rocprofv3
 # FETCH_SIZE + WRITE_SIZE, scaled by what the same counters read for the plain copy kernel of known size
 # (profiles/moe_layer_mixtral_hbm_traffic.txt).  None where it has not been measured.
-TRAFFIC_BYTES_PER_LAUNCH = {"mixtral": 5269622426}
+TRAFFIC_BYTES_PER_LAUNCH = {"mixtral": 5227968600}
 
 WORKLOADS = {
     # name: (tokens, hidden, experts, topk, ffn, dtype, routing)
