@@ -574,7 +574,9 @@ __global__ __launch_bounds__(256) void unpermute_grad_kernel(
                         if (c >= vecs) continue;
                         const S *xp = permuted + static_cast<int64_t>(d[j]) * hidden + static_cast<int64_t>(c) * VEC;
                         if constexpr (VEC * sizeof(S) == 16) {
-                            *reinterpret_cast<v16 *>(x[j][u]) = *reinterpret_cast<const v16 *>(xp);
+                            // plain loads measured faster with two slots per token, non-temporal ones with more
+                            if constexpr (JB == 2) *reinterpret_cast<v16 *>(x[j][u]) = *reinterpret_cast<const v16 *>(xp);
+                            else *reinterpret_cast<v16 *>(x[j][u]) = MS_NT_LOAD(reinterpret_cast<const v16 *>(xp));
                         } else {
 #pragma unroll
                             for (int e = 0; e < VEC; ++e) x[j][u][e] = xp[e];
