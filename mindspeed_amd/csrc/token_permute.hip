@@ -633,6 +633,39 @@ __global__ void copy_tail_kernel(const unsigned char *src, unsigned char *dst, s
     if (i < end) dst[i] = src[i];
 }
 
+// ---- pieces shared by the one-launch permute kernels ---------------------------------------
+// The first eight vectors of a thread's source row, as unconditional loads from clamped positions: straight-line
+// code, so that the compiler's waits for loads issued before these can leave them in flight.
+template <typename VecT>
+__device__ __forceinline__ void prefetch_row(VecT (&v)[8], const VecT *__restrict__ src, int lane, int lanes,
+                                             int vecs_per_row) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+}
+
+// Write one source row to the rows listed in dest[0 .. count) (entries outside [0, limit) are skipped), `lanes`
+// threads per row, eight vectors per thread at a time; v holds the row's first eight vectors already.
+template <typename VecT>
+__device__ __forceinline__ void scatter_row(VecT (&v)[8], const VecT *__restrict__ src, VecT *__restrict__ permuted,
+                                            const int *dest, int count, int limit, int lane, int lanes,
+                                            int vecs_per_row) {
+    for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
+        if (c0 != lane) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
+        }
+        for (int j = 0; j < count; ++j) {
+            const int row = dest[j];
+            if (static_cast<unsigned>(row) >= static_cast<unsigned>(limit)) continue;   // dropped
+            VecT *dst = permuted + static_cast<int64_t>(row) * vecs_per_row;
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + c0 + u * lanes);
+        }
+    }
+}
+
 // ---- sort and row scatter in one launch ------------------------------------------------
 constexpr int kFusedMaxBins = 16;     // one private LDS counter column per thread and bin; more bins: two launches
 constexpr int kFusedMaxLocal = 4096;  // flat positions of one workgroup whose rows are handed over through LDS
@@ -743,8 +776,7 @@ __global__ __launch_bounds__(1024) void permute_fused_kernel(
     if (tid < 64) own = idx[min(p0 + tid, n - 1)];
     VecT v[8];   // the first vectors of this thread's row; unconditional loads from clamped positions, so that
                  // the waits for the indices above can leave these in flight
-#pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+    prefetch_row(v, src, lane, lanes, vecs_per_row);
     __syncthreads();
     unsigned bad = 0;
     fused_add<IdxT, NB, false>(table, raw, 0, n, p0, nbins - 1, bad);
@@ -789,22 +821,7 @@ __global__ __launch_bounds__(1024) void permute_fused_kernel(
     __syncthreads();
 
     if (!mover) return;
-    const int *d = dest + local_row * topk;
-    for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
-        if (c0 != lane) {
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
-        }
-        for (int j = 0; j < topk; ++j) {
-            const int row = d[j];
-            if (static_cast<unsigned>(row) >= static_cast<unsigned>(num_out)) continue;   // dropped
-            VecT *dst = permuted + static_cast<int64_t>(row) * vecs_per_row;
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + c0 + u * lanes);
-        }
-    }
+    scatter_row(v, src, permuted, dest + local_row * topk, topk, num_out, lane, lanes, vecs_per_row);
 }
 
 // The one-launch permute for more than kFusedMaxBins bins (up to MS_MAX_EXPERTS, which is what a call without
@@ -841,8 +858,7 @@ __global__ __launch_bounds__(1024) void permute_fused_bins_kernel(
     if (tid < 64) own = idx[min(p0 + tid, n - 1)];
     VecT v[8];   // first vectors of this thread's row: unconditional loads from clamped positions, in flight
                  // while the keys are counted
-#pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+    prefetch_row(v, src, lane, lanes, vecs_per_row);
     __syncthreads();
     unsigned unused = 0;
     for (int c = 0; c < n; c += kFusedKeys * nthreads) {
@@ -885,22 +901,7 @@ __global__ __launch_bounds__(1024) void permute_fused_bins_kernel(
     }
     __syncthreads();
     if (!mover) return;
-    const int *d = dest + local_row * topk;
-    for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
-        if (c0 != lane) {
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
-        }
-        for (int j = 0; j < topk; ++j) {
-            const int row = d[j];
-            if (static_cast<unsigned>(row) >= static_cast<unsigned>(num_out)) continue;   // dropped
-            VecT *dst = permuted + static_cast<int64_t>(row) * vecs_per_row;
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + c0 + u * lanes);
-        }
-    }
+    scatter_row(v, src, permuted, dest + local_row * topk, topk, num_out, lane, lanes, vecs_per_row);
 }
 
 // Stable scatter and row movement in one launch, behind the histogram launch of the multi-block sort (any bin
@@ -971,8 +972,7 @@ __global__ __launch_bounds__(1024) void permute_scatter_rows_kernel(
     // counting needs - loads retire in order, so an earlier request would stall the counting until the rows are
     // in - and in flight during the scan and the ranking below.
     VecT v[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+    prefetch_row(v, src, lane, lanes, vecs_per_row);
     if constexpr (!SCANNED) {
         __syncthreads();
         int carry = 0;
@@ -1012,22 +1012,7 @@ __global__ __launch_bounds__(1024) void permute_scatter_rows_kernel(
     }
     __syncthreads();
     if (!mover) return;
-    const int *d = dest + local_row * topk;
-    for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
-        if (c0 != lane) {
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
-        }
-        for (int j = 0; j < topk; ++j) {
-            const int row = d[j];
-            if (static_cast<unsigned>(row) >= static_cast<unsigned>(num_out)) continue;   // dropped
-            VecT *dst = permuted + static_cast<int64_t>(row) * vecs_per_row;
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + c0 + u * lanes);
-        }
-    }
+    scatter_row(v, src, permuted, dest + local_row * topk, topk, num_out, lane, lanes, vecs_per_row);
 }
 
 // ---- routing-map (mask) mode ----------------------------------------------------------
@@ -1152,8 +1137,7 @@ __global__ __launch_bounds__(1024) void routing_map_fused_kernel(
     if (tid < 64) own0 = map[min(split + tid, n - 1)];
     v16 v[8];                                   // the first vectors of this thread's row (clamped, unconditional)
     if (tokens != nullptr) {
-#pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+        prefetch_row(v, src, lane, lanes, vecs_per_row);
     }
     __syncthreads();
     mask_vector_add(table, w, tid * 16, tid < nvec ? 1 : 0, split, E);
@@ -1204,22 +1188,7 @@ __global__ __launch_bounds__(1024) void routing_map_fused_kernel(
     }
     __syncthreads();
     if (!mover) return;
-    const int *d = rows + local_row * E;
-    for (int c0 = lane; c0 < vecs_per_row; c0 += 8 * lanes) {
-        if (c0 != lane) {
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (c0 + u * lanes < vecs_per_row) v[u] = src[c0 + u * lanes];
-        }
-        for (int j = 0; j < E; ++j) {
-            const int row = d[j];
-            if (static_cast<unsigned>(row) >= static_cast<unsigned>(num_rows)) continue;
-            v16 *dst = permuted + static_cast<int64_t>(row) * vecs_per_row;
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (c0 + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + c0 + u * lanes);
-        }
-    }
+    scatter_row(v, src, permuted, rows + local_row * E, E, num_rows, lane, lanes, vecs_per_row);
 }
 
 // Mask mode for any expert count (no drop-and-pad), two launches.  The map is cut into chunks of `chunk` tokens
@@ -1288,8 +1257,7 @@ __global__ __launch_bounds__(1024) void routing_map_ranked_kernel(
     // are in - and in flight during the scan and the ranking below, which work out of LDS.
     VecT v[8];
     if (tokens != nullptr) {
-#pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = src[min(lane + u * lanes, vecs_per_row - 1)];
+        prefetch_row(v, src, lane, lanes, vecs_per_row);
     }
     __syncthreads();
     int carry = 0;
@@ -1326,21 +1294,7 @@ __global__ __launch_bounds__(1024) void routing_map_ranked_kernel(
     }
     __syncthreads();
     if (!mover) return;
-    const int mine = ntok[local_row];
-    const int *d = list + local_row * E;
-    for (int cv = lane; cv < vecs_per_row; cv += 8 * lanes) {
-        if (cv != lane) {
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (cv + u * lanes < vecs_per_row) v[u] = src[cv + u * lanes];
-        }
-        for (int j = 0; j < mine; ++j) {
-            VecT *dst = permuted + static_cast<int64_t>(d[j]) * vecs_per_row;
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (cv + u * lanes < vecs_per_row) MS_NT_STORE(v[u], dst + cv + u * lanes);
-        }
-    }
+    scatter_row(v, src, permuted, list + local_row * E, ntok[local_row], num_rows, lane, lanes, vecs_per_row);
 }
 
 // ---- host helpers -------------------------------------------------------------------
