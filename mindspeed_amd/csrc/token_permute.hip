@@ -1,10 +1,17 @@
 // MoE token permute / unpermute for gfx950 (MI355X).
 //
 // permute  = stable counting sort of the flattened expert ids (wavefront-ballot
-//            match, per-wave histogram rows, LDS prefix scan, no atomics, so
-//            the order is deterministic) followed by a coalesced 16-byte row
+//            match, histogram rows in LDS, LDS prefix scan; no atomic decides an
+//            order, so the result is deterministic) and a coalesced 16-byte row
 //            scatter that reads every token row once and writes its topk
-//            copies.
+//            copies.  Up to 16384 positions both happen in one launch
+//            (permute_fused_kernel for at most 16 bins, permute_fused_bins_kernel
+//            for more); beyond that a histogram launch is followed by
+//            permute_scatter_rows_kernel.  The routing-map form counts per expert
+//            column instead of sorting (routing_map_fused_kernel,
+//            routing_map_hist_kernel + routing_map_ranked_kernel); the separate
+//            sort_* / permute_rows kernels serve what is left (no rows to move,
+//            drop-and-pad, shapes the fused forms do not take).
 // unpermute = per-token top-k gather with fp32 accumulation in registers and
 //            one rounding; its backward scatters prob-scaled rows and reduces
 //            the per-(token, slot) dot products for grad_probs.
