@@ -676,23 +676,57 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
             }
         }
     } else {
-        const bool full_cols = col0 + BN <= col_end;
+        // fp32 output or fp32 `+=`: an accumulator register holds four consecutive columns of one row, so written
+        // straight from the registers one instruction would touch 32 rows with 32 bytes each.  Instead each
+        // wavefront stages one 32-row strip of its block at a time in its own LDS region (row pitch WC + 4
+        // floats) and moves it as whole row segments: WC * 4 contiguous bytes per row, 16 bytes per lane.
+        constexpr int SPF = WC + 4;              // floats per staged row
+        static_assert(32 * SPF * 4 <= kStagePerWave, "staging region too small");
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_s_barrier();          // every wavefront is done reading the operand stages
+        float *stg = reinterpret_cast<float *>(lds + wave * kStagePerWave);
+        constexpr int LPR = WC / 4;            // lanes per row (4 columns = 16 bytes each)
+        constexpr int RPP = 64 / LPR;          // rows per pass
+        const int c4 = (lane % LPR) * 4;
+        const int col = col0 + wn * WC + c4;
+        const bool col_ok = col < col_end;     // cols is a multiple of 4 on this path
+        float *cbase = static_cast<float *>(p.c) + tc.e.c_off + col;
+        const float *lbase = static_cast<const float *>(p.c) + tc.e.c_off + (col_ok ? col : col_end - 4);   // always inside the row
+        constexpr int NP = 32 / RPP;           // passes per strip
+        // `+=`: the old values of strip i + 1 are requested while strip i is staged and written, from clamped
+        // (always valid) addresses, so that a whole strip's loads are in flight at a time
+        f32x4 old[2][NP];
+        auto load_old = [&](f32x4 (&dst)[NP], int i) {
+#pragma unroll
+            for (int pass = 0; pass < NP; ++pass) {
+                int row = row0 + wm * WR + i * 32 + pass * RPP + lane / LPR;
+                row = row < row_end ? row : row_end - 1;
+                dst[pass] = *reinterpret_cast<const f32x4 *>(lbase + static_cast<int64_t>(row) * ldc);
+            }
+        };
+        if constexpr (OUT == ACC_F32) load_old(old[0], 0);
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const int row = row0 + wm * WR + i * 32 + (lane & 31);
-            if (row >= row_end) continue;
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const int col = col0 + wn * WC + j * 32 + 8 * q + 4 * hi;
-                    if (!full_cols && col >= col_end) continue;   // cols is a multiple of 4 on this path
-                    float *c = static_cast<float *>(p.c) + tc.e.c_off + static_cast<int64_t>(row) * ldc + col;
-                    f32x4 o = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                    if constexpr (OUT == ACC_F32) o += *reinterpret_cast<f32x4 *>(c);
-                    *reinterpret_cast<f32x4 *>(c) = o;
+                    const f32x4 o = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    *reinterpret_cast<f32x4 *>(stg + (lane & 31) * SPF + j * 32 + 8 * q + 4 * hi) = o;
                 }
+            if constexpr (OUT == ACC_F32) {
+                if (i + 1 < TM) load_old(old[(i + 1) & 1], i + 1);
             }
+            __builtin_amdgcn_s_waitcnt(0xC07F);    // own writes only: the region is private to this wavefront
+#pragma unroll
+            for (int pass = 0; pass < NP; ++pass) {
+                const int r = pass * RPP + lane / LPR;
+                const int row = row0 + wm * WR + i * 32 + r;
+                f32x4 o = *reinterpret_cast<const f32x4 *>(stg + r * SPF + c4);
+                if constexpr (OUT == ACC_F32) o += old[i & 1][pass];
+                if (col_ok && row < row_end) *reinterpret_cast<f32x4 *>(cbase + static_cast<int64_t>(row) * ldc) = o;
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);    // the strip has been read before the next one overwrites it
         }
     }
 }
