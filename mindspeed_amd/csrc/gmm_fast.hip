@@ -701,7 +701,7 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
             for (int pass = 0; pass < NP; ++pass) {
                 int row = row0 + wm * WR + i * 32 + pass * RPP + lane / LPR;
                 row = row < row_end ? row : row_end - 1;
-                dst[pass] = *reinterpret_cast<const f32x4 *>(lbase + static_cast<int64_t>(row) * ldc);
+                dst[pass] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(lbase + static_cast<int64_t>(row) * ldc));
             }
         };
         if constexpr (OUT == ACC_F32) load_old(old[0], 0);
@@ -724,7 +724,7 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
                 const int row = row0 + wm * WR + i * 32 + r;
                 f32x4 o = *reinterpret_cast<const f32x4 *>(stg + r * SPF + c4);
                 if constexpr (OUT == ACC_F32) o += old[i & 1][pass];
-                if (col_ok && row < row_end) *reinterpret_cast<f32x4 *>(cbase + static_cast<int64_t>(row) * ldc) = o;
+                if (col_ok && row < row_end) __builtin_nontemporal_store(o, reinterpret_cast<f32x4 *>(cbase + static_cast<int64_t>(row) * ldc));
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);    // the strip has been read before the next one overwrites it
         }
