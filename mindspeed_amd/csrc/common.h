@@ -37,6 +37,10 @@ void set_error(const char *fmt, ...);
         }                                                                         \
     } while (0)
 
+// hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes), issued once per kernel and device
+// (and again only if a larger size is asked for); later calls are a table lookup.  Returns a hipError_t.
+hipError_t set_max_dynamic_lds(const void *fn, int bytes);
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int dtype_size(int dtype) { return dtype == MS_FP32 ? 4 : 2; }

@@ -450,12 +450,12 @@ int current_device_cus() {
     return cached[dev];
 }
 
-size_t table_bytes(int64_t num_groups) {
+constexpr size_t table_bytes(int64_t num_groups) {
     return sizeof(TileTable) + static_cast<size_t>(2 * num_groups + 2) * sizeof(GroupEntry);   // full + tail entries
 }
 // workspace = tile table, then (8-byte aligned) room for the per-group weight offsets of the list form
-size_t offsets_pos(int64_t num_groups) { return (table_bytes(num_groups) + 7) & ~static_cast<size_t>(7); }
-size_t workspace_need(int64_t num_groups) { return offsets_pos(num_groups) + kMaxWeightList * sizeof(int64_t); }
+constexpr size_t offsets_pos(int64_t num_groups) { return (table_bytes(num_groups) + 7) & ~static_cast<size_t>(7); }
+constexpr size_t workspace_need(int64_t num_groups) { return offsets_pos(num_groups) + kMaxWeightList * sizeof(int64_t); }
 
 template <int DT, int OUT>
 int launch16(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red, unsigned grid) {
@@ -464,7 +464,7 @@ int launch16(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red, un
     else if (a_red) fn = reinterpret_cast<const void *>(&gmm16_kernel<DT, true, false, OUT>);
     else if (b_red) fn = reinterpret_cast<const void *>(&gmm16_kernel<DT, false, true, OUT>);
     else fn = reinterpret_cast<const void *>(&gmm16_kernel<DT, false, false, OUT>);
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes16);
+    hipError_t e = set_max_dynamic_lds(fn, kLdsBytes16);
     MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "ms_gmm: hipFuncSetAttribute: %s", hipGetErrorString(e));
     GmmArgs copy = args;
     void *kargs[] = {&copy};
@@ -661,9 +661,15 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     const bool a_truly_contig = a_is_red ? a_stride_red == 1 : a_stride_row == 1;
     const bool b_truly_contig = b_is_red ? b_stride_red == 1 : b_stride_col == 1;
     bool fast = args.a_vec_ok && args.b_vec_ok && args.c_vec_ok && a_truly_contig && b_truly_contig;
-    if (a_is_red) fast = fast && red_total % 8 == 0 && group_type == 0; else fast = fast && out_rows % 8 == 0 && out_rows >= 8;
+    // An operand that is contiguous along its outer dim is fetched in whole 8-index chunks clamped to the end of the
+    // tile's row range, so that range must be the full, 8-aligned extent: for x that only holds when the split is on
+    // the reduction dim (with a split on rows the groups' row ranges start and end anywhere).
+    if (a_is_red) fast = fast && red_total % 8 == 0 && group_type == 0;
+    else fast = fast && group_type == 2 && out_rows % 8 == 0 && out_rows >= 8;
     if (b_is_red) fast = fast && red_total % 8 == 0 && group_type == 0; else fast = fast && n % 8 == 0 && n >= 8;
-    fast = fast && n % 4 == 0 && (out_dtype != MS_FP32 || reinterpret_cast<uintptr_t>(y) % 16 == 0);
+    // the epilogue writes 16 bytes per lane: 8 columns of a 16-bit output, 4 of an fp32 one
+    fast = fast && (out_dtype == MS_FP32 ? n % 4 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0
+                                         : n % 8 == 0 && aligned16(y) && y_stride_row % 8 == 0);
     // per-lane global offsets are 32-bit byte offsets inside one 256 x 64 operand tile
     const int64_t a_span = a_is_red ? 256 * a_stride_row : 64 * a_stride_red;
     const int64_t b_span = b_is_red ? 256 * b_stride_col : 64 * b_stride_red;

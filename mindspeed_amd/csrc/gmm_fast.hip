@@ -254,12 +254,11 @@ struct RingOperand {
     // tile costs the same number of transfers whatever it holds: the wait counters of the K loop rely on that.
     // Written as inline assembly on purpose: the compiler then does not know that LDS is being written
     // behind its back and leaves all waiting on these transfers to the explicit s_waitcnt of the K loop
-    // (it would otherwise drain them before every transposing LDS read).  M0 carries the LDS address; no
-    // other code in these kernels uses M0.
+    // (it would otherwise drain them before every transposing LDS read).  M0 carries the LDS address (declared as clobbered).
     __device__ __forceinline__ void request(int i, const char *base, unsigned dst, int nvalid, const char *zeros) const {
         const char *src = key[i] < nvalid ? base + off[i] : zeros;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                     :: "s"(dst + i * 1024), "v"(src) : "memory");
+                     :: "s"(dst + i * 1024), "v"(src) : "memory", "m0");
     }
 
     // Fragment t of 16-wide slice kk of the tile at `tile`.
@@ -757,7 +756,7 @@ int launch_fast(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red,
     int lds_bytes = 2 * ((a_red ? kRedTileBytes : kOuterTileBytes) + (b_red ? kRedTileBytes : kOuterTileBytes));
     if ((OUT == OUT_SAME || OUT == OUT_SWIGLU || OUT == OUT_SWIGLU_GRAD) && lds_bytes < kStageBytes) lds_bytes = kStageBytes;
     if (!a_red && !b_red && lds_bytes < kRingBytes) lds_bytes = kRingBytes;   // use_ring<false, false>()
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    hipError_t e = set_max_dynamic_lds(fn, lds_bytes);
     MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "ms_gmm: hipFuncSetAttribute: %s", hipGetErrorString(e));
     GmmArgs copy = args;
     void *kargs[] = {&copy};

@@ -89,6 +89,8 @@ GMM_CASES = [
     (300, 64, 256, 1, "equal"),
     (96, 1000, 24, 4, "equal"),           # long reduction, narrow output
     (37, 19, 23, 5, "random"),            # tiny and odd: element-wise paths
+    (96, 20, 16, 3, "random"),            # dX writes 20 columns: a multiple of 4 but not of 8
+    (256, 72, 44, 2, "equal"),            # forward writes 44 columns (n % 8 == 4) from vector-aligned operands
 ]
 
 
@@ -144,6 +146,28 @@ def test_transposed_weight_view_and_raw_module(device):
     assert rel_l2(y, exp) <= 1e-2 and rel_l2(dx[0], e_dx) <= 1e-2 and rel_l2(dw[0], e_dw) <= 1e-2 and dbias == []
     dx2, dw2, _ = mod.npu_gmm_backward_fusion([gy.to(device)], [w], cum, 0)
     assert torch.equal(dx2[0], dx[0]) and dw2 == []
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_row_contiguous_x_with_split_on_rows(dtype, device):
+    """x handed over as the transposed view of a [K, M] buffer (unit stride along its rows) with a split on rows:
+    groups of 3, 13 and 0 rows start and end off the 8-row chunks such an operand is fetched in."""
+    gen = torch.Generator().manual_seed(11)
+    counts = torch.tensor([3, 13, 0, 40, 8, 64])
+    M, K, N = int(counts.sum()), 64, 96
+    xt = torch.randn(K, M, generator=gen).to(dtype)
+    w = (torch.randn(len(counts), K, N, generator=gen) * 0.05).to(dtype)
+    exp = O.gmm(xt.t().contiguous(), w, counts, 0, 1)
+    x_view = xt.to(device).t()
+    assert x_view.stride(0) == 1
+    got = ops.npu_gmm_v2(x_view, w.to(device), group_list=counts.to(device), group_type=0)
+    assert rel_l2(got, exp) <= TOL[dtype]
+    got = ops.npu_gmm(x_view, w.to(device), group_list=torch.cumsum(counts, 0).tolist(), group_type=0)
+    assert rel_l2(got, exp) <= TOL[dtype]
+    # the same view with a transposed weight view (both operands off their usual layouts)
+    wt = w.transpose(1, 2).contiguous().to(device).transpose(1, 2)
+    got = ops.npu_gmm_v2(x_view, wt, group_list=counts.to(device), group_type=0)
+    assert rel_l2(got, exp) <= TOL[dtype]
 
 
 def test_rows_past_last_offset_are_zero(device):
