@@ -190,6 +190,21 @@ int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_strid
            int group_type, int64_t num_groups, int64_t m, int64_t k, int64_t n, int dtype,
            int out_dtype, int accumulate, void *workspace, size_t workspace_bytes);
 
+/* ms_gmm for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the same arguments without the workspace pair, the same
+ * kernels and results.  It has no counterpart in the reference, whose shims always draw a workspace
+ * from the framework's allocator.  The tile table lives in a fixed device array inside the library
+ * (about 120 KB per GPU, held until the process ends), which bounds num_groups to 1024; more groups
+ * report MS_ERR_UNSUPPORTED.  The call allocates and frees nothing.  The first call on a device looks
+ * the array's address up (hipGetSymbolAddress), so make that call outside a graph capture.  All calls
+ * on one GPU share the array: calls that may overlap on one GPU (different streams, different
+ * threads) race on it and must be ordered by the caller. */
+int ms_gmm_noalloc(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1,
+                   const void *weight, int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1,
+                   void *y, int64_t y_stride_row, const int64_t *group_list, int group_list_type,
+                   int group_type, int64_t num_groups, int64_t m, int64_t k, int64_t n, int dtype,
+                   int out_dtype, int accumulate);
+
 /* First grouped matmul of an expert MLP with the SwiGLU (x per-row probability) activation fused into
  * its epilogue: the op sequence fc1 = gmm(x, w1); act = (silu(gate) * up * probs).to(dtype) of
  * mindspeed/core/transformer/moe/moe_feature/gmm/experts.py:113-127 (activation: :41-44) in one launch.

@@ -44,6 +44,8 @@ _SIGNATURES = {
     "ms_gmm_workspace_size": [_i64, _i64, _int, ctypes.POINTER(_size_t)],
     "ms_gmm": [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _i64, _i64, _i64, _c_void_p, _i64, _c_void_p, _int, _int,
                _i64, _i64, _i64, _i64, _int, _int, _int, _c_void_p, _size_t],
+    "ms_gmm_noalloc": [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _i64, _i64, _i64, _c_void_p, _i64, _c_void_p, _int,
+                       _int, _i64, _i64, _i64, _i64, _int, _int, _int],
     "ms_gmm_swiglu": [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _i64, _i64, _i64, _c_void_p, _i64, _c_void_p, _i64,
                       _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _int, _c_void_p, _size_t],
     "ms_gmm_swiglu_grad_workspace_size": [_i64, _i64, _i64, ctypes.POINTER(_size_t)],

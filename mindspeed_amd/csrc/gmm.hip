@@ -17,6 +17,8 @@
 //     reduction dim transposed in registers on their way to LDS), same
 //     256x256x64 tile and 4x4 v_mfma_f32_32x32x16 per wavefront; and
 //     gmm32_kernel for fp32 inputs (v_mfma_f32_32x32x2f32, 128x128x8 tiles).
+#include <mutex>
+
 #include "gmm_common.h"
 
 namespace ms {
@@ -708,6 +710,51 @@ extern "C" int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int6
     return gmm_impl(stream, x, x_stride0, x_stride1, weight, w_stride_group, w_stride0, w_stride1, y, y_stride_row,
                     group_list, group_list_type, group_type, num_groups, m, k, n, dtype, out_dtype, accumulate,
                     workspace, workspace_bytes, nullptr, false);
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------------------------
+// The tile table that ms_gmm takes through its workspace argument lives here in a fixed device array, one copy per
+// GPU.  In host code the array's name is only a handle for hipGetSymbolAddress; kernels get the address that call
+// returned, looked up once per device.
+constexpr int kNoAllocMaxGroups = 1024;
+constexpr size_t kScratchBytes = (workspace_need(kNoAllocMaxGroups) + 255) & ~static_cast<size_t>(255);
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+int scratch_of_current_device(void **out) {
+    static std::mutex mu;
+    static void *ptrs[kMaxDevices] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    MS_REQUIRE(e == hipSuccess, MS_ERR_HIP, "ms_gmm_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+    MS_REQUIRE(dev >= 0 && dev < kMaxDevices, MS_ERR_UNSUPPORTED, "ms_gmm_noalloc: device ordinal %d outside [0, %d)", dev,
+               kMaxDevices);
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptrs[dev] == nullptr) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        MS_REQUIRE(e == hipSuccess && p != nullptr, MS_ERR_HIP, "ms_gmm_noalloc: hipGetSymbolAddress: %s",
+                   hipGetErrorString(e));
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return MS_OK;
+}
+}  // namespace
+
+extern "C" int ms_gmm_noalloc(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1, const void *weight,
+                              int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1, void *y, int64_t y_stride_row,
+                              const int64_t *group_list, int group_list_type, int group_type, int64_t num_groups,
+                              int64_t m, int64_t k, int64_t n, int dtype, int out_dtype, int accumulate) {
+    MS_REQUIRE(num_groups >= 1 && num_groups <= kNoAllocMaxGroups, MS_ERR_UNSUPPORTED,
+               "ms_gmm_noalloc: num_groups %lld outside [1, %d] (the fixed tile-table buffer holds no more; use ms_gmm "
+               "with a caller-provided workspace beyond that)", (long long)num_groups, kNoAllocMaxGroups);
+    void *table = nullptr;
+    if (int rc = scratch_of_current_device(&table)) return rc;
+    return gmm_impl(stream, x, x_stride0, x_stride1, weight, w_stride_group, w_stride0, w_stride1, y, y_stride_row,
+                    group_list, group_list_type, group_type, num_groups, m, k, n, dtype, out_dtype, accumulate, table,
+                    kScratchBytes, nullptr, false);
 }
 
 extern "C" int ms_gmm_swiglu(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1, const void *weight,
