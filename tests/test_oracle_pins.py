@@ -340,3 +340,35 @@ def test_routing_map_mode_agrees_with_index_mode():
     out_idx = O.unpermute(p_idx, sorted_flat, topk_probs)
     out_map = O.unpermute_routing_map(p_map, sidx, tokens.shape, probs, rmap)
     assert torch.allclose(out_idx, out_map, rtol=1e-6, atol=1e-6)
+
+
+def test_row_reference_agrees_with_oracle_autograd():
+    """The per-row / per-block fp32 evaluation used by the full-size GPU tests (tests/layer_rowref.py) against
+    autograd through the whole-layer oracle on a small fp32 configuration: every token, every weight block."""
+    from layer_rowref import RowRef
+
+    cfg = dict(T=96, H=40, E=6, K=3, F=24)
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn(cfg["T"], cfg["H"], generator=gen)
+    p, idx = O.route_topk(torch.randn(cfg["T"], cfg["E"], generator=gen), cfg["K"])
+    idx[idx == 4] = 5                                                    # expert 4 gets no rows
+    w1 = torch.randn(cfg["E"], cfg["H"], 2 * cfg["F"], generator=gen) * 0.3
+    w2 = torch.randn(cfg["E"], cfg["F"], cfg["H"], generator=gen) * 0.3
+    gy = torch.randn(cfg["T"], cfg["H"], generator=gen)
+    leaves = [t.clone().requires_grad_(True) for t in (x, p, w1, w2)]
+    out = O.moe_layer(leaves[0], idx, leaves[1], leaves[2], leaves[3])
+    dx, dp, dw1, dw2 = torch.autograd.grad(out, leaves, gy)
+
+    ref = RowRef(cfg, x, p, idx, w1, w2, gy)
+    tokens = list(range(cfg["T"]))
+    r_out, r_dx, r_dp = ref.token_refs(tokens)
+    assert torch.allclose(r_out, out.detach(), rtol=1e-5, atol=1e-5)
+    assert torch.allclose(r_dx, dx, rtol=1e-5, atol=1e-5)
+    assert torch.allclose(r_dp, dp, rtol=1e-5, atol=1e-5)
+    ks, fs, hs = torch.arange(3, 29), torch.arange(5, 24), torch.arange(0, 40, 3)
+    for e in range(cfg["E"]):
+        g, u, d2 = ref.dw_blocks(e, ks, fs, hs)
+        assert torch.allclose(g, dw1[e][ks][:, fs], rtol=1e-5, atol=1e-5)
+        assert torch.allclose(u, dw1[e][ks][:, cfg["F"] + fs], rtol=1e-5, atol=1e-5)
+        assert torch.allclose(d2, dw2[e][fs][:, hs], rtol=1e-5, atol=1e-5)
+    assert ref.counts[4] == 0 and torch.count_nonzero(dw1[4]) == 0
