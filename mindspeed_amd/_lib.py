@@ -114,8 +114,9 @@ def index_code(dtype: torch.dtype, what: str) -> int:
 
 
 def require_device(t: torch.Tensor, what: str):
-    """The kernels run on a HIP device only."""
-    if t.device.type != "cuda":
+    """The kernels run on a HIP device only (meta tensors pass: they only propagate shapes through the
+    dispatcher ops' fake kernels)."""
+    if t.device.type not in ("cuda", "meta"):
         raise RuntimeError(
             f"{what} is on {t.device}: mindspeed_amd ops run hand-written HIP kernels and need tensors on an "
             "MI355X (torch device type 'cuda' on ROCm); there is no CPU fallback.")

@@ -1,0 +1,324 @@
+"""The C-ABI kernel calls as dispatcher ops (namespace ``mindspeed_amd``).
+
+Every op here is one call of an entry point of ``libmindspeed_amd.so`` on tensors that the Python surface has
+already validated.  Registering them with the dispatcher, each with a device kernel and a fake (meta) kernel
+that only computes output shapes, is what lets the Python surface above them (autograd Functions, the
+``mindspeed::npu_gmm`` ops) run on meta / fake tensors, i.e. be traced by ``torch.compile`` and shape-propagated
+without touching the GPU — the job the reference's ``Meta`` registrations do for its ops
+(mindspeed/op_builder/gmm_builder.py:101-106,141-146).
+
+There is no CPU kernel: on CPU tensors the ops raise.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from .. import _lib, flop_counter
+
+_LIB = torch.library.Library("mindspeed_amd", "DEF")
+
+
+def _define(schema, device_fn, fake_fn):
+    name = schema.split("(")[0]
+    _LIB.define(schema)
+    _LIB.impl(name, device_fn, "CUDA")
+    torch.library.register_fake(f"mindspeed_amd::{name}", fake_fn, lib=_LIB)
+
+    def _no_cpu(*args, **kwargs):
+        raise RuntimeError(f"mindspeed_amd::{name} runs hand-written HIP kernels and needs tensors on an MI355X "
+                           "(torch device type 'cuda' on ROCm); there is no CPU fallback.")
+    _LIB.impl(name, _no_cpu, "CPU")
+
+
+# ---- grouped matmul ----------------------------------------------------------------------------------------
+def _gmm_dims(x, weight, group_list, group_type):
+    """(m, k, n, weight strides (group, red, col), output shape) of one grouped matmul."""
+    num_groups = group_list.numel()
+    if group_type == 0:
+        m, k = x.shape
+        n = weight.size(2)
+        return m, k, n, (weight.stride(0), weight.stride(1), weight.stride(2)), (m, n)
+    k, m = x.shape
+    n = weight.size(1)
+    return m, k, n, (0, weight.stride(0), weight.stride(1)), (num_groups, k, n)
+
+
+def _gmm_launch(x, weight, group_list, group_type, group_list_type, out, accumulate):
+    lib = _lib.load()
+    dev = x.device
+    dtype = _lib.dtype_code(x.dtype, "x")
+    m, k, n, w_strides, _ = _gmm_dims(x, weight, group_list, group_type)
+    num_groups = group_list.numel()
+    out_dtype = _lib.MS_FP32 if out.dtype == torch.float32 else dtype
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(lib.ms_gmm_workspace_size(num_groups, m, group_type, ctypes.byref(nbytes)), "ms_gmm_workspace_size")
+    ws = _lib.workspace(nbytes.value, dev)
+    # kernel flavour by operand layout: NN (forward), NT (weight read transposed: dX), TN (dW)
+    if group_type == 2:
+        kind = "gmm_dw"
+    elif w_strides[1] == 1 and w_strides[2] != 1:
+        kind = "gmm_dx"
+    else:
+        kind = "gmm_fwd"
+    with torch.cuda.device(dev), flop_counter.op(kind, flop_counter.gmm_flops(m, k, n), "flop", dev):
+        _lib.check(lib.ms_gmm(
+            _lib.stream_ptr(dev), _lib.ptr(x), x.stride(0), x.stride(1), _lib.ptr(weight), *w_strides,
+            _lib.ptr(out), n, _lib.ptr(group_list), group_list_type, group_type, num_groups, m, k, n, dtype, out_dtype,
+            1 if accumulate else 0, _lib.ptr(ws), ws.numel()), "ms_gmm")
+
+
+def _gmm(x, weight, group_list, group_type, group_list_type):
+    out = torch.empty(_gmm_dims(x, weight, group_list, group_type)[4], dtype=x.dtype, device=x.device)
+    _gmm_launch(x, weight, group_list, group_type, group_list_type, out, False)
+    return out
+
+
+def _gmm_fake(x, weight, group_list, group_type, group_list_type):
+    return x.new_empty(_gmm_dims(x, weight, group_list, group_type)[4])
+
+
+def _gmm_out(x, weight, group_list, group_type, group_list_type, out, accumulate):
+    _gmm_launch(x, weight, group_list, group_type, group_list_type, out, accumulate)
+
+
+_define("gmm(Tensor x, Tensor weight, Tensor group_list, int group_type, int group_list_type) -> Tensor",
+        _gmm, _gmm_fake)
+_define("gmm_out(Tensor x, Tensor weight, Tensor group_list, int group_type, int group_list_type, "
+        "Tensor(a!) out, bool accumulate) -> ()", _gmm_out, lambda *a: None)
+
+
+# ---- token permute / unpermute -----------------------------------------------------------------------------
+def _permute_shapes(tokens, indices, num_out, num_experts, want_sorted, want_counts):
+    num_tokens, hidden = tokens.shape
+    topk = 1 if indices.dim() == 1 else indices.size(1)
+    return ((num_out, hidden), num_tokens * topk, num_out if want_sorted else 0,
+            num_experts if (want_counts and num_experts > 0) else 0, topk)
+
+
+def _permute(tokens, indices, num_out, num_experts, want_sorted, want_counts):
+    lib = _lib.load()
+    dev = tokens.device
+    pshape, flat, nsorted, ncounts, topk = _permute_shapes(tokens, indices, num_out, num_experts, want_sorted,
+                                                           want_counts)
+    num_tokens, hidden = tokens.shape
+    row_id_map = torch.empty(flat, dtype=torch.int32, device=dev)
+    permuted = torch.empty(pshape, dtype=tokens.dtype, device=dev)
+    sorted_idx = torch.empty(nsorted, dtype=torch.int32, device=dev)
+    counts = torch.empty(ncounts, dtype=torch.int64, device=dev)
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(lib.ms_moe_token_permute_workspace_size(num_tokens, topk, num_experts, ctypes.byref(nbytes)),
+               "ms_moe_token_permute_workspace_size")
+    ws = _lib.workspace(nbytes.value, dev)
+    work = flop_counter.permute_bytes(num_tokens, topk, hidden, tokens.element_size(), indices.element_size(), num_out)
+    with torch.cuda.device(dev), flop_counter.op("permute", work, "byte", dev):
+        _lib.check(lib.ms_moe_token_permute(
+            _lib.stream_ptr(dev), _lib.ptr(tokens), _lib.ptr(indices), _lib.index_code(indices.dtype, "indices"),
+            num_tokens, topk, hidden, _lib.dtype_code(tokens.dtype, "tokens"), num_out, num_experts,
+            _lib.ptr(permuted), _lib.ptr(row_id_map), _lib.ptr(sorted_idx) if want_sorted else None,
+            _lib.ptr(counts) if ncounts else None, _lib.ptr(ws), ws.numel()), "ms_moe_token_permute")
+    return permuted, row_id_map, sorted_idx, counts
+
+
+def _permute_fake(tokens, indices, num_out, num_experts, want_sorted, want_counts):
+    pshape, flat, nsorted, ncounts, _ = _permute_shapes(tokens, indices, num_out, num_experts, want_sorted, want_counts)
+    return (tokens.new_empty(pshape), tokens.new_empty(flat, dtype=torch.int32),
+            tokens.new_empty(nsorted, dtype=torch.int32), tokens.new_empty(ncounts, dtype=torch.int64))
+
+
+_define("moe_token_permute(Tensor tokens, Tensor indices, int num_out, int num_experts, bool want_sorted, "
+        "bool want_counts) -> (Tensor, Tensor, Tensor, Tensor)", _permute, _permute_fake)
+
+
+def _permute_grad(grad_permuted, row_id_map, num_tokens, topk):
+    lib = _lib.load()
+    dev = grad_permuted.device
+    hidden = grad_permuted.size(1)
+    grad_tokens = torch.empty((num_tokens, hidden), dtype=grad_permuted.dtype, device=dev)
+    work = flop_counter.permute_grad_bytes(num_tokens, topk, hidden, grad_permuted.element_size(), grad_permuted.size(0))
+    with torch.cuda.device(dev), flop_counter.op("permute_grad", work, "byte", dev):
+        _lib.check(lib.ms_moe_token_permute_grad(
+            _lib.stream_ptr(dev), _lib.ptr(grad_permuted), _lib.ptr(row_id_map), num_tokens, topk, hidden,
+            _lib.dtype_code(grad_permuted.dtype, "grad_permuted_tokens"), grad_permuted.size(0),
+            _lib.ptr(grad_tokens)), "ms_moe_token_permute_grad")
+    return grad_tokens
+
+
+_define("moe_token_permute_grad(Tensor grad_permuted, Tensor row_id_map, int num_tokens, int topk) -> Tensor",
+        _permute_grad, lambda g, r, num_tokens, topk: g.new_empty((num_tokens, g.size(1))))
+
+
+def _unpermute(permuted, row_id_map, probs, num_tokens, topk):
+    lib = _lib.load()
+    dev = permuted.device
+    hidden = permuted.size(1)
+    out = torch.empty((num_tokens, hidden), dtype=permuted.dtype, device=dev)
+    work = flop_counter.unpermute_bytes(num_tokens, topk, hidden, permuted.element_size(), permuted.size(0))
+    with torch.cuda.device(dev), flop_counter.op("unpermute", work, "byte", dev):
+        _lib.check(lib.ms_moe_token_unpermute(
+            _lib.stream_ptr(dev), _lib.ptr(permuted), _lib.ptr(row_id_map), _lib.ptr(probs), num_tokens, topk, hidden,
+            _lib.dtype_code(permuted.dtype, "permuted_tokens"), permuted.size(0), _lib.ptr(out)),
+            "ms_moe_token_unpermute")
+    return out
+
+
+_define("moe_token_unpermute(Tensor permuted, Tensor row_id_map, Tensor? probs, int num_tokens, int topk) -> Tensor",
+        _unpermute, lambda p, r, probs, num_tokens, topk: p.new_empty((num_tokens, p.size(1))))
+
+
+def _unpermute_grad(permuted, grad_out, row_id_map, probs, num_tokens, topk, num_rows):
+    """``permuted`` may be an empty tensor when there are no probabilities (it is only read for their gradient)."""
+    lib = _lib.load()
+    dev = grad_out.device
+    hidden = grad_out.size(1)
+    rows = num_rows
+    grad_permuted = torch.empty((rows, hidden), dtype=grad_out.dtype, device=dev)
+    grad_probs = torch.empty_like(probs) if probs is not None else torch.empty(0, dtype=grad_out.dtype, device=dev)
+    mapped = min(rows, num_tokens * topk)
+    if rows > mapped:
+        grad_permuted.zero_()
+    work = flop_counter.unpermute_grad_bytes(num_tokens, topk, hidden, grad_out.element_size(), rows, probs is not None)
+    with torch.cuda.device(dev), flop_counter.op("unpermute_grad", work, "byte", dev):
+        _lib.check(lib.ms_moe_token_unpermute_grad(
+            _lib.stream_ptr(dev), _lib.ptr(permuted) if probs is not None else None, _lib.ptr(grad_out),
+            _lib.ptr(row_id_map), _lib.ptr(probs), num_tokens, topk, hidden,
+            _lib.dtype_code(grad_out.dtype, "unpermuted_tokens_grad"), mapped, _lib.ptr(grad_permuted),
+            _lib.ptr(grad_probs) if probs is not None else None), "ms_moe_token_unpermute_grad")
+    return grad_permuted, grad_probs
+
+
+def _unpermute_grad_fake(permuted, grad_out, row_id_map, probs, num_tokens, topk, num_rows):
+    return (grad_out.new_empty((num_rows, grad_out.size(1))),
+            torch.empty_like(probs) if probs is not None else grad_out.new_empty(0))
+
+
+_define("moe_token_unpermute_grad(Tensor permuted, Tensor grad_out, Tensor row_id_map, Tensor? probs, "
+        "int num_tokens, int topk, int num_rows) -> (Tensor, Tensor)", _unpermute_grad, _unpermute_grad_fake)
+
+
+# ---- SwiGLU --------------------------------------------------------------------------------------------------
+def _swiglu(x2, probs):
+    lib = _lib.load()
+    rows, two_ffn = x2.shape
+    ffn = two_ffn // 2
+    y = torch.empty((rows, ffn), dtype=x2.dtype, device=x2.device)
+    p_code = _lib.dtype_code(probs.dtype, "probs") if probs is not None else 0
+    with torch.cuda.device(x2.device), flop_counter.op(
+            "swiglu", flop_counter.swiglu_bytes(rows, ffn, x2.element_size()), "byte", x2.device):
+        _lib.check(lib.ms_swiglu(_lib.stream_ptr(x2.device), _lib.ptr(x2), _lib.ptr(probs), p_code, rows, ffn,
+                                 _lib.dtype_code(x2.dtype, "x"), _lib.ptr(y)), "ms_swiglu")
+    return y
+
+
+_define("swiglu(Tensor x, Tensor? probs) -> Tensor", _swiglu, lambda x2, probs: x2.new_empty((x2.size(0), x2.size(1) // 2)))
+
+
+def _swiglu_grad(g, x2, probs):
+    lib = _lib.load()
+    rows, two_ffn = x2.shape
+    ffn = two_ffn // 2
+    gx = torch.empty_like(x2)
+    gp = torch.empty_like(probs) if probs is not None else torch.empty(0, dtype=x2.dtype, device=x2.device)
+    p_code = _lib.dtype_code(probs.dtype, "probs") if probs is not None else 0
+    with torch.cuda.device(x2.device), flop_counter.op(
+            "swiglu_grad", flop_counter.swiglu_bytes(rows, ffn, x2.element_size(), True), "byte", x2.device):
+        _lib.check(lib.ms_swiglu_grad(_lib.stream_ptr(x2.device), _lib.ptr(g), _lib.ptr(x2), _lib.ptr(probs), p_code,
+                                      rows, ffn, _lib.dtype_code(x2.dtype, "x"), _lib.ptr(gx),
+                                      _lib.ptr(gp) if probs is not None else None), "ms_swiglu_grad")
+    return gx, gp
+
+
+_define("swiglu_grad(Tensor grad_y, Tensor x, Tensor? probs) -> (Tensor, Tensor)", _swiglu_grad,
+        lambda g, x2, probs: (torch.empty_like(x2), torch.empty_like(probs) if probs is not None else x2.new_empty(0)))
+
+
+
+# ---- routing-map (mask) form ---------------------------------------------------------------------------------
+def _routing_map_permute(tokens, routing_map, num_rows, drop_and_pad, want_counts):
+    """``tokens`` may be None (maps only).  Returns (permuted or empty, row_id_map, sorted_flat, counts or empty)."""
+    lib = _lib.load()
+    dev = routing_map.device
+    num_tokens, num_experts = routing_map.shape
+    row_id_map = torch.empty(num_tokens * num_experts, dtype=torch.int32, device=dev)
+    sorted_flat = torch.empty(num_rows, dtype=torch.int32, device=dev)
+    counts = torch.empty(num_experts if want_counts else 0, dtype=torch.int64, device=dev)
+    hidden, dtype_code, elem = 1, _lib.MS_FP32, 0
+    if tokens is not None:
+        hidden = tokens.size(1)
+        dtype_code = _lib.dtype_code(tokens.dtype, "tokens")
+        elem = tokens.element_size()
+        permuted = torch.empty((num_rows, hidden), dtype=tokens.dtype, device=dev)
+    else:
+        permuted = torch.empty(0, dtype=torch.float32, device=dev)
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(lib.ms_moe_routing_map_workspace_size(num_tokens, num_experts, int(drop_and_pad), ctypes.byref(nbytes)),
+               "ms_moe_routing_map_workspace_size")
+    ws = _lib.workspace(nbytes.value, dev)
+    work = (num_tokens * hidden * elem + num_rows * hidden * elem if tokens is not None else 0) \
+        + num_tokens * num_experts * (1 + 4) + num_rows * 4
+    with torch.cuda.device(dev), flop_counter.op("permute", work, "byte", dev):
+        _lib.check(lib.ms_moe_routing_map_permute(
+            _lib.stream_ptr(dev), _lib.ptr(tokens), _lib.ptr(routing_map), num_tokens, num_experts, hidden, dtype_code,
+            num_rows, int(drop_and_pad), _lib.ptr(permuted) if tokens is not None else None, _lib.ptr(row_id_map),
+            _lib.ptr(sorted_flat), _lib.ptr(counts) if want_counts else None, _lib.ptr(ws), ws.numel()),
+            "ms_moe_routing_map_permute")
+    return permuted, row_id_map, sorted_flat, counts
+
+
+def _routing_map_permute_fake(tokens, routing_map, num_rows, drop_and_pad, want_counts):
+    num_tokens, num_experts = routing_map.shape
+    permuted = tokens.new_empty((num_rows, tokens.size(1))) if tokens is not None \
+        else routing_map.new_empty(0, dtype=torch.float32)
+    return (permuted, routing_map.new_empty(num_tokens * num_experts, dtype=torch.int32),
+            routing_map.new_empty(num_rows, dtype=torch.int32),
+            routing_map.new_empty(num_experts if want_counts else 0, dtype=torch.int64))
+
+
+_define("routing_map_permute(Tensor? tokens, Tensor routing_map, int num_rows, bool drop_and_pad, bool want_counts) "
+        "-> (Tensor, Tensor, Tensor, Tensor)", _routing_map_permute, _routing_map_permute_fake)
+
+
+def _routing_map_probs(sorted_flat, probs, num_experts):
+    """(permuted_probs or empty, sorted token ids int64)."""
+    lib = _lib.load()
+    dev = sorted_flat.device
+    num_rows = sorted_flat.numel()
+    permuted_probs = torch.empty(num_rows if probs is not None else 0,
+                                 dtype=probs.dtype if probs is not None else torch.float32, device=dev)
+    sorted_indices = torch.empty(num_rows, dtype=torch.int64, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.ms_moe_routing_map_probs(
+            _lib.stream_ptr(dev), _lib.ptr(sorted_flat), num_rows, num_experts, _lib.ptr(probs),
+            _lib.dtype_code(probs.dtype, "probs") if probs is not None else 0,
+            _lib.ptr(permuted_probs) if probs is not None else None, _lib.ptr(sorted_indices)),
+            "ms_moe_routing_map_probs")
+    return permuted_probs, sorted_indices
+
+
+def _routing_map_probs_fake(sorted_flat, probs, num_experts):
+    n = sorted_flat.numel()
+    pp = probs.new_empty(n) if probs is not None else sorted_flat.new_empty(0, dtype=torch.float32)
+    return pp, sorted_flat.new_empty(n, dtype=torch.int64)
+
+
+_define("routing_map_probs(Tensor sorted_flat, Tensor? probs, int num_experts) -> (Tensor, Tensor)",
+        _routing_map_probs, _routing_map_probs_fake)
+
+
+def _routing_map_probs_grad(row_id_map, grad_permuted_probs, num_tokens, num_experts):
+    lib = _lib.load()
+    dev = row_id_map.device
+    probs_grad = torch.empty((num_tokens, num_experts), dtype=grad_permuted_probs.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.ms_moe_routing_map_probs_grad(
+            _lib.stream_ptr(dev), _lib.ptr(row_id_map), row_id_map.numel(), _lib.ptr(grad_permuted_probs),
+            _lib.dtype_code(grad_permuted_probs.dtype, "probs"), grad_permuted_probs.numel(), _lib.ptr(probs_grad)),
+            "ms_moe_routing_map_probs_grad")
+    return probs_grad
+
+
+_define("routing_map_probs_grad(Tensor row_id_map, Tensor grad_permuted_probs, int num_tokens, int num_experts) -> Tensor",
+        _routing_map_probs_grad, lambda r, g, num_tokens, num_experts: g.new_empty((num_tokens, num_experts)))
+
+K = torch.ops.mindspeed_amd

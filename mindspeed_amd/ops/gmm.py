@@ -17,6 +17,7 @@ import os
 import torch
 
 from .. import _lib, flop_counter
+from ._kernels import K
 from .npu_groupmatmul_add import npu_groupmatmul_add_fp32
 
 __all__ = ["npu_gmm", "npu_gmm_v2", "GMMFunction"]
@@ -48,11 +49,10 @@ def gmm_raw(x, weight, group_list, group_type, group_list_type, out=None, accumu
     ``out``: optional preallocated contiguous result (fp32, or x's dtype); fp32 with ``accumulate`` adds the
     result in place.
     """
-    lib = _lib.load()
     _lib.require_device(x, "x")
     _lib.require_device(weight, "weight")
     dev = x.device
-    dtype = _lib.dtype_code(x.dtype, "x")
+    _lib.dtype_code(x.dtype, "x")
     if weight.dtype != x.dtype:
         raise TypeError(f"x and weight must have the same dtype, got {x.dtype} and {weight.dtype}")
     gl = _group_list_tensor(group_list, dev)
@@ -82,30 +82,13 @@ def gmm_raw(x, weight, group_list, group_type, group_list_type, out=None, accumu
     else:
         raise ValueError(f"group_type must be 0 or 2, got {group_type}")
     if out is None:
-        out = torch.empty(out_shape, dtype=x.dtype, device=dev)
-        out_dtype = dtype
-    else:
-        numel = out_shape[0] * out_shape[1] * (out_shape[2] if len(out_shape) == 3 else 1)
-        if out.dtype not in (torch.float32, x.dtype) or not out.is_contiguous() or out.numel() != numel:
-            raise ValueError("out must be a contiguous tensor of the result's size, fp32 or of x's dtype")
-        if accumulate and out.dtype != torch.float32:
-            raise ValueError("accumulate needs an fp32 out")
-        out_dtype = _lib.MS_FP32 if out.dtype == torch.float32 else dtype
-    nbytes = ctypes.c_size_t(0)
-    _lib.check(lib.ms_gmm_workspace_size(num_groups, m, group_type, ctypes.byref(nbytes)), "ms_gmm_workspace_size")
-    ws = _lib.workspace(nbytes.value, dev)
-    # kernel flavour by operand layout: NN (forward), NT (weight read transposed: dX), TN (dW)
-    if group_type == 2:
-        kind = "gmm_dw"
-    elif w_strides[1] == 1 and w_strides[2] != 1:
-        kind = "gmm_dx"
-    else:
-        kind = "gmm_fwd"
-    with torch.cuda.device(dev), flop_counter.op(kind, flop_counter.gmm_flops(m, k, n), "flop", dev):
-        _lib.check(lib.ms_gmm(
-            _lib.stream_ptr(dev), _lib.ptr(x), x.stride(0), x.stride(1), _lib.ptr(weight), *w_strides,
-            _lib.ptr(out), n, _lib.ptr(gl), group_list_type, group_type, num_groups, m, k, n, dtype, out_dtype,
-            1 if accumulate else 0, _lib.ptr(ws), ws.numel()), "ms_gmm")
+        return K.gmm(x, weight, gl, group_type, group_list_type)
+    numel = out_shape[0] * out_shape[1] * (out_shape[2] if len(out_shape) == 3 else 1)
+    if out.dtype not in (torch.float32, x.dtype) or not out.is_contiguous() or out.numel() != numel:
+        raise ValueError("out must be a contiguous tensor of the result's size, fp32 or of x's dtype")
+    if accumulate and out.dtype != torch.float32:
+        raise ValueError("accumulate needs an fp32 out")
+    K.gmm_out(x, weight, gl, group_type, group_list_type, out, bool(accumulate))
     return out
 
 
@@ -179,16 +162,16 @@ def _side_stream(device) -> torch.cuda.Stream:
 
 
 class _beside:
-    """``with _beside(device) as side:`` runs the body on the side stream after everything queued so far on the
+    """``with _beside(tensor) as side:`` runs the body on the side stream after everything queued so far on the
     current stream; ``side.join()`` (call it after queueing the main-stream work that should overlap)
     makes the current stream wait for the body.  Results of the body should live in memory that was
     allocated on the caller's stream beforehand.  Without overlap (disabled,
     or while ops are being event-timed one by one) the body simply runs on the current stream."""
 
-    def __init__(self, device):
-        self.device = device
-        self.active = OVERLAP_WGRAD and not flop_counter.timing_active()
-        self.main = torch.cuda.current_stream(device)
+    def __init__(self, like: torch.Tensor):
+        device = like.device
+        self.active = OVERLAP_WGRAD and not flop_counter.timing_active() and not _tracing(like)
+        self.main = torch.cuda.current_stream(device) if self.active else None
         self.side = _side_stream(device) if self.active else None
         self.ctx = None
 
@@ -241,7 +224,7 @@ class _RawGmmModule:
         w = weight[0]
         num_groups = len(group_list) if not isinstance(group_list, torch.Tensor) else group_list.numel()
         dw = torch.empty((num_groups, x[0].size(-1), grad[0].size(-1)), dtype=x[0].dtype, device=x[0].device)
-        with _beside(grad[0].device) as side:
+        with _beside(grad[0]) as side:
             gmm_raw(x[0].transpose(-1, -2), grad[0], group_list, 2, glt, out=dw)
         dx = gmm_raw(grad[0], w.transpose(-1, -2), group_list, 0, glt)
         side.join()
@@ -262,18 +245,26 @@ class _Builder:
         return self._module
 
 
-def check_optional_tensor(tensor, device, name):
-    if not isinstance(tensor, (torch.Tensor, type(None))):
-        raise TypeError(f"{name} must be a torch.Tensor or None, got {type(tensor)}.")
-    if isinstance(tensor, torch.Tensor) and tensor.device != device:
-        raise RuntimeError(
-            f"Expected all tensors to be on the same device, but found at least two devices, "
-            f"{device}(arg0) and {tensor.device}({name})!")
+def _tracing(t: torch.Tensor) -> bool:
+    """True when ``t`` is a meta / fake tensor or a compiler is tracing: no kernel runs then, so there is nothing
+    to overlap and no stream to fork."""
+    return t.device.type == "meta" or torch.compiler.is_compiling() or \
+        isinstance(t, torch._subclasses.fake_tensor.FakeTensor)
 
 
 class GMMFunction(torch.autograd.Function):
+    """Autograd node of ``npu_gmm`` / ``npu_gmm_v2`` (mindspeed/ops/gmm.py:20-99).
+
+    ``apply(original_weight, x, weight, bias, group_args)`` with ``group_args = (group_list, group_type,
+    gemm_fusion, group_list_type, group_list_data_type)``; gradients ``(None, dx, dw, dbias, None)``.  A list
+    ``group_list`` (data type 0) rides on the context, a tensor one is saved with the other tensors.
+    """
     builder = _Builder()
     builder2 = _Builder()
+
+    @staticmethod
+    def _module(group_list_type):
+        return (GMMFunction.builder if group_list_type == 0 else GMMFunction.builder2).load()
 
     @staticmethod
     def forward(ctx, original_weight, x, weight, bias, group_args):
@@ -282,51 +273,37 @@ class GMMFunction(torch.autograd.Function):
             raise ValueError("Bias is not supported to compute gradient!")
         if (x.requires_grad or weight.requires_grad) and group_type != 0:
             raise ValueError("group_type must be zero to compute gradients of x and weight!")
-        bias = [] if bias is None else [bias]
-        module = GMMFunction.builder.load() if group_list_type == 0 else GMMFunction.builder2.load()
-        outputs = module.npu_gmm([x], [weight], bias, group_list, group_type, group_list_type)
-        if group_list_data_type == 0:
-            ctx.save_for_backward(x, weight, original_weight)
-            ctx.group_list = group_list
-        else:
-            ctx.save_for_backward(x, weight, group_list, original_weight)
+        (y,) = GMMFunction._module(group_list_type).npu_gmm(
+            [x], [weight], [] if bias is None else [bias], group_list, group_type, group_list_type)
+        list_form = group_list_data_type == 0
+        ctx.save_for_backward(x, weight, original_weight, *(() if list_form else (group_list,)))
+        ctx.group_list = group_list if list_form else None
         ctx.gemm_fusion = gemm_fusion
         ctx.group_list_type = group_list_type
-        ctx.group_list_data_type = group_list_data_type
-        return outputs[0]
+        return y
 
     @staticmethod
-    def backward(ctx, grad_outputs):
-        if ctx.group_list_data_type == 0:
-            x, weight, original_weight = ctx.saved_tensors
-            group_list = ctx.group_list
-        else:
-            x, weight, group_list, original_weight = ctx.saved_tensors
-        module = GMMFunction.builder.load() if ctx.group_list_type == 0 else GMMFunction.builder2.load()
-
-        if ctx.gemm_fusion:
-            with _beside(grad_outputs.device) as side:
-                if ctx.group_list_type == 0:
-                    cumulative = group_list
-                else:
-                    cumulative = torch.cumsum(group_list, dim=0)
-                npu_groupmatmul_add_fp32(x, grad_outputs, cumulative, original_weight.main_grad)
-            dx, _, dbias = module.npu_gmm_backward_fusion([grad_outputs], [weight], group_list, ctx.group_list_type)
-            side.join()
-            dbias = None if len(dbias) == 0 else dbias[0]
-            if hasattr(original_weight, "grad_added_to_main_grad"):
-                if getattr(weight, "zero_out_wgrad", False):
-                    grad_weight = torch.zeros(weight.shape, dtype=x.dtype, device=x.device, requires_grad=False)
-                else:
-                    grad_weight = torch.empty(weight.shape, dtype=x.dtype, device=x.device, requires_grad=False)
-                original_weight.grad_added_to_main_grad = True
-            else:
-                grad_weight = None
-            return None, dx[0], grad_weight, dbias, None
-
-        dx, dw, dbias = module.npu_gmm_backward([grad_outputs], [x], [weight], group_list, ctx.group_list_type)
-        dbias = None if len(dbias) == 0 else dbias[0]
-        return None, dx[0], dw[0], dbias, None
+    def backward(ctx, grad_y):
+        x, weight, original_weight, *rest = ctx.saved_tensors
+        group_list = rest[0] if rest else ctx.group_list
+        module = GMMFunction._module(ctx.group_list_type)
+        if not ctx.gemm_fusion:
+            (dx,), (dw,), dbias = module.npu_gmm_backward([grad_y], [x], [weight], group_list, ctx.group_list_type)
+            return None, dx, dw, (dbias[0] if dbias else None), None
+        # gemm_fusion (gmm.py:56-89): the weight gradient is added into original_weight.main_grad (fp32) by the
+        # accumulate form of the dW product, here on the side stream beside dX; what autograd gets for the weight is
+        # a placeholder (zeros if the parameter asks for it) and the flag the optimizer wrapper looks at is set.
+        with _beside(grad_y) as side:
+            offsets = group_list if ctx.group_list_type == 0 else torch.cumsum(group_list, dim=0)
+            npu_groupmatmul_add_fp32(x, grad_y, offsets, original_weight.main_grad)
+        (dx,), _, dbias = module.npu_gmm_backward_fusion([grad_y], [weight], group_list, ctx.group_list_type)
+        side.join()
+        placeholder = None
+        if hasattr(original_weight, "grad_added_to_main_grad"):
+            make = torch.zeros if getattr(weight, "zero_out_wgrad", False) else torch.empty
+            placeholder = make(weight.shape, dtype=x.dtype, device=x.device, requires_grad=False)
+            original_weight.grad_added_to_main_grad = True
+        return None, dx, placeholder, (dbias[0] if dbias else None), None
 
 
 def npu_gmm_param_verification(x, weight, *, bias=None, group_list=None, group_type=0, group_list_type=0):
@@ -406,8 +383,11 @@ def _npu_gmm_v2(original_weight, x, weight, *, bias=None, group_list=None, group
 
 for _name, _fn in (("npu_gmm.List", _npu_gmm), ("npu_gmm.Tensor", _npu_gmm), ("npu_gmm_v2.Tensor", _npu_gmm_v2)):
     if _name in _DEFINED:
-        # The implementation is an autograd.Function over the raw kernel call,
-        # so it is registered as a composite that autograd sees through.
+        # The implementation is an autograd.Function over dispatcher ops that carry their own device and fake
+        # (meta) kernels (ops/_kernels.py), so it is registered as a composite: autograd sees through it, and on
+        # meta / fake tensors it decomposes into those ops and yields the output shape the reference's explicit
+        # Meta registrations compute (mindspeed/op_builder/gmm_builder.py:101-106,141-146).  torch refuses a
+        # direct Meta kernel next to a composite one.
         _LIBRARY.impl(_name, _fn, "CompositeImplicitAutograd")
 
 

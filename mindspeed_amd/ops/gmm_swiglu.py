@@ -95,7 +95,7 @@ class GmmSwigluFunction(torch.autograd.Function):
         dx = dw = None
         if ctx.needs_input_grad[1]:
             dw = torch.empty(weight.shape, dtype=weight.dtype, device=dev)
-            with _beside(dev) as side:
+            with _beside(d_fc1) as side:
                 gmm_raw(x.t(), d_fc1, gl, 2, glt, out=dw)
             if ctx.needs_input_grad[0]:
                 dx = gmm_raw(d_fc1, weight.transpose(1, 2), gl, 0, glt)
@@ -204,7 +204,7 @@ class GroupedMLPFunction(torch.autograd.Function):
         # everything the side stream writes is allocated here, on the caller's stream
         dw1 = torch.empty(w1.shape, dtype=w1.dtype, device=dev) if ctx.needs_input_grad[1] else None
         dw2 = torch.empty(w2.shape, dtype=w2.dtype, device=dev) if ctx.needs_input_grad[2] else None
-        side = _beside(dev)
+        side = _beside(dy)
         with side:                                   # dW2 needs only act and dy
             if dw2 is not None:
                 gmm_raw(act.t(), dy, gl, 2, glt, out=dw2)

@@ -8,7 +8,8 @@ from __future__ import annotations
 
 import torch
 
-from .. import _lib, flop_counter
+from .. import _lib
+from ._kernels import K
 
 __all__ = ["npu_moe_token_permute", "moe_token_permute_with_aux"]
 
@@ -37,7 +38,6 @@ def _actual_num_out(num_out_tokens, flatten_size):
 
 
 def _permute_forward(tokens, indices, num_out, num_experts, want_sorted, want_counts):
-    lib = _lib.load()
     tokens = tokens.contiguous()
     indices = indices.contiguous()
     num_tokens, hidden = tokens.shape
@@ -48,26 +48,12 @@ def _permute_forward(tokens, indices, num_out, num_experts, want_sorted, want_co
     hint = 0 if num_experts is None else int(num_experts)
     if hint > _lib.MS_MAX_EXPERTS:
         raise RuntimeError(f"num_experts {hint} exceeds the sort's key range {_lib.MS_MAX_EXPERTS}")
-    dev = tokens.device
-    row_id_map = torch.empty(flat, dtype=torch.int32, device=dev)
-    permuted = torch.empty((num_out, hidden), dtype=tokens.dtype, device=dev)
-    sorted_idx = torch.empty(num_out, dtype=torch.int32, device=dev) if want_sorted else None
-    counts = torch.empty(hint, dtype=torch.int64, device=dev) if (want_counts and hint > 0) else None
     if hidden == 0:
         raise RuntimeError("tokens must have a non-empty hidden dimension")
-    import ctypes
-    nbytes = ctypes.c_size_t(0)
-    _lib.check(lib.ms_moe_token_permute_workspace_size(num_tokens, topk, hint, ctypes.byref(nbytes)),
-               "ms_moe_token_permute_workspace_size")
-    ws = _lib.workspace(nbytes.value, dev)
-    work = flop_counter.permute_bytes(num_tokens, topk, hidden, tokens.element_size(), indices.element_size(), num_out)
-    with torch.cuda.device(dev), flop_counter.op("permute", work, "byte", dev):
-        _lib.check(lib.ms_moe_token_permute(
-            _lib.stream_ptr(dev), _lib.ptr(tokens), _lib.ptr(indices), _lib.index_code(indices.dtype, "indices"),
-            num_tokens, topk, hidden, _lib.dtype_code(tokens.dtype, "tokens"), num_out, hint,
-            _lib.ptr(permuted), _lib.ptr(row_id_map), _lib.ptr(sorted_idx), _lib.ptr(counts),
-            _lib.ptr(ws), ws.numel()), "ms_moe_token_permute")
-    return permuted, row_id_map, sorted_idx, counts, topk
+    permuted, row_id_map, sorted_idx, counts = K.moe_token_permute(
+        tokens, indices, num_out, hint, bool(want_sorted), bool(want_counts and hint > 0))
+    return (permuted, row_id_map, sorted_idx if want_sorted else None,
+            counts if (want_counts and hint > 0) else None, topk)
 
 
 class _MoeTokenPermute(torch.autograd.Function):
@@ -98,18 +84,7 @@ class _MoeTokenPermute(torch.autograd.Function):
         if grad_permuted.dim() != 2:
             raise RuntimeError("The dims of input grad_permuted_tokens should be 2 dimensional, "
                                f"but got {grad_permuted.dim()}-dimensional.")
-        grad_permuted = grad_permuted.contiguous()
-        lib = _lib.load()
-        dev = grad_permuted.device
-        hidden = grad_permuted.size(1)
-        grad_tokens = torch.empty((ctx.num_tokens, hidden), dtype=grad_permuted.dtype, device=dev)
-        work = flop_counter.permute_grad_bytes(ctx.num_tokens, ctx.topk, hidden, grad_permuted.element_size(),
-                                               grad_permuted.size(0))
-        with torch.cuda.device(dev), flop_counter.op("permute_grad", work, "byte", dev):
-            _lib.check(lib.ms_moe_token_permute_grad(
-                _lib.stream_ptr(dev), _lib.ptr(grad_permuted), _lib.ptr(row_id_map), ctx.num_tokens, ctx.topk,
-                hidden, _lib.dtype_code(grad_permuted.dtype, "grad_permuted_tokens"), grad_permuted.size(0),
-                _lib.ptr(grad_tokens)), "ms_moe_token_permute_grad")
+        grad_tokens = K.moe_token_permute_grad(grad_permuted.contiguous(), row_id_map, ctx.num_tokens, ctx.topk)
         return grad_tokens, None, None, None, None, None
 
 

@@ -8,7 +8,8 @@ from __future__ import annotations
 
 import torch
 
-from .. import _lib, flop_counter
+from .. import _lib
+from ._kernels import K
 
 __all__ = ["npu_moe_token_unpermute"]
 
@@ -39,7 +40,6 @@ def _check_forward(permuted_tokens, sorted_indices, probs, padded_mode):
 class _MoeTokenUnpermute(torch.autograd.Function):
     @staticmethod
     def forward(ctx, permuted_tokens, sorted_indices, probs):
-        lib = _lib.load()
         permuted_tokens = permuted_tokens.contiguous()
         sorted_indices = sorted_indices.contiguous()
         topk = 1 if probs is None else probs.size(1)
@@ -50,16 +50,7 @@ class _MoeTokenUnpermute(torch.autograd.Function):
             probs = probs.contiguous()
             if probs.size(0) != num_tokens:
                 raise RuntimeError(f"probs has {probs.size(0)} rows, expected {num_tokens}")
-        hidden = permuted_tokens.size(1)
-        dev = permuted_tokens.device
-        out = torch.empty((num_tokens, hidden), dtype=permuted_tokens.dtype, device=dev)
-        work = flop_counter.unpermute_bytes(num_tokens, topk, hidden, permuted_tokens.element_size(),
-                                            permuted_tokens.size(0))
-        with torch.cuda.device(dev), flop_counter.op("unpermute", work, "byte", dev):
-            _lib.check(lib.ms_moe_token_unpermute(
-                _lib.stream_ptr(dev), _lib.ptr(permuted_tokens), _lib.ptr(sorted_indices), _lib.ptr(probs),
-                num_tokens, topk, hidden, _lib.dtype_code(permuted_tokens.dtype, "permuted_tokens"),
-                permuted_tokens.size(0), _lib.ptr(out)), "ms_moe_token_unpermute")
+        out = K.moe_token_unpermute(permuted_tokens, sorted_indices, probs, num_tokens, topk)
         ctx.save_for_backward(permuted_tokens, sorted_indices, probs)  # npu_moe_token_unpermute.cpp:117
         ctx.topk = topk
         ctx.num_tokens = num_tokens
@@ -68,27 +59,15 @@ class _MoeTokenUnpermute(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         permuted_tokens, sorted_indices, probs = ctx.saved_tensors
-        lib = _lib.load()
         if grad_out.dim() != 2:
             raise RuntimeError("The dims of input unpermuted_tokens_grad should be 2 dimensional, "
                                f"but got {grad_out.dim()}-dimensional.")
-        grad_out = grad_out.contiguous()
-        dev = grad_out.device
-        hidden = permuted_tokens.size(1)
-        grad_permuted = torch.empty_like(permuted_tokens)  # npu_moe_token_unpermute.cpp:140
-        grad_probs = torch.empty_like(probs) if probs is not None else None  # :141
-        need_rows = ctx.num_tokens * ctx.topk
-        if permuted_tokens.size(0) > need_rows:
-            grad_permuted.zero_()
-        work = flop_counter.unpermute_grad_bytes(ctx.num_tokens, ctx.topk, hidden, grad_out.element_size(),
-                                                 permuted_tokens.size(0), probs is not None)
-        with torch.cuda.device(dev), flop_counter.op("unpermute_grad", work, "byte", dev):
-            _lib.check(lib.ms_moe_token_unpermute_grad(
-                _lib.stream_ptr(dev), _lib.ptr(permuted_tokens), _lib.ptr(grad_out), _lib.ptr(sorted_indices),
-                _lib.ptr(probs), ctx.num_tokens, ctx.topk, hidden,
-                _lib.dtype_code(permuted_tokens.dtype, "permuted_tokens"), min(permuted_tokens.size(0), need_rows),
-                _lib.ptr(grad_permuted), _lib.ptr(grad_probs)), "ms_moe_token_unpermute_grad")
-        return grad_permuted, None, grad_probs
+        # grad_permuted has the shape of permuted_tokens, grad_probs that of probs (npu_moe_token_unpermute.cpp:140-141);
+        # rows of permuted_tokens that no (token, slot) pair maps to get zeros
+        grad_permuted, grad_probs = K.moe_token_unpermute_grad(
+            permuted_tokens, grad_out.contiguous(), sorted_indices, probs, ctx.num_tokens, ctx.topk,
+            permuted_tokens.size(0))
+        return grad_permuted, None, (grad_probs if probs is not None else None)
 
 
 def npu_moe_token_unpermute(permuted_tokens: torch.Tensor, sorted_indices: torch.Tensor,

@@ -43,6 +43,9 @@ unpermute_routing_map         pairs incl. drop-and-pad, equality with the index
                               ``moe_utils.permute/unpermute`` (a dependency that
                               is not vendored in the reference tree), restated
                               from its published source.
+fused_permute_routing_map     pinned: hand-typed table of result dtypes for every
+                              (tokens, probs) dtype pair, values equal to the
+                              plain permutation cast to those dtypes.
 fused-op output conventions   PARITY UNPINNED: what the closed vendor kernels
   (second output of           ``aclnnMoeTokenPermute`` / ``aclnnGroupedMatmul``
   npu_moe_token_permute,      really return for dropped rows, rows past the
@@ -59,7 +62,7 @@ __all__ = [
     "permute_backward", "unpermute_backward", "grouped_matmul", "gmm_split",
     "gmm", "gmm_backward", "groupmatmul_add_fp32", "swiglu", "swiglu_backward",
     "sort_chunks_by_idxs", "experts_computation", "moe_layer", "route_topk",
-    "permute_routing_map", "unpermute_routing_map",
+    "permute_routing_map", "fused_permute_routing_map", "unpermute_routing_map",
 ]
 
 
@@ -429,6 +432,25 @@ def permute_routing_map(tokens, routing_map, probs=None, num_out_tokens=None, dr
             # same expression as mindspeed/core/transformer/moe/moe_feature/overlap/token_dispatcher.py:451-453
             permuted_probs = probs.T.contiguous().masked_select(rm)
     permuted = tokens.index_select(0, sorted_indices)
+    return permuted, permuted_probs, sorted_indices
+
+
+def fused_permute_routing_map(tokens, routing_map, probs=None, num_out_tokens=None, drop_and_pad=False):
+    """The reference's ``permute`` hook with ``fused=True``
+    (mindspeed/core/fusions/fused_moe_permute.py:17-47,58-63): when exactly one of ``tokens`` / ``probs`` is
+    fp32, both are promoted to fp32, permuted, and *both* results are cast to the dtype of the operand that was
+    not fp32 (``convert_tensors_to_fp32_if_needed`` / ``restore_original_dtype``).  Any other dtype pair, and a
+    call without ``probs``, goes through unchanged."""
+    original = None
+    if isinstance(tokens, torch.Tensor) and isinstance(probs, torch.Tensor) and \
+            ((tokens.dtype == torch.float32) ^ (probs.dtype == torch.float32)):
+        original = probs.dtype if tokens.dtype == torch.float32 else tokens.dtype
+        tokens, probs = tokens.to(torch.float32), probs.to(torch.float32)
+    permuted, permuted_probs, sorted_indices = permute_routing_map(tokens, routing_map, probs, num_out_tokens,
+                                                                   drop_and_pad)
+    if original is not None:
+        permuted = permuted.to(original)
+        permuted_probs = permuted_probs.to(original) if permuted_probs is not None else None
     return permuted, permuted_probs, sorted_indices
 
 

@@ -40,6 +40,7 @@ CASES = [
     (512, 64, 8, 96, torch.bfloat16, torch.bfloat16, ()),         # T*E = 32768: multi-block sort
     (4096, 8, 2, 512, torch.bfloat16, torch.float32, ()),         # Mixtral routing at reduced hidden
     (2000, 130, 4, 32, torch.bfloat16, torch.float32, (129,)),    # > 64 experts, ragged
+    (200, 8, 2, 64, torch.float32, torch.bfloat16, ()),           # fp32 tokens next to 16-bit probabilities
 ]
 
 
@@ -50,20 +51,26 @@ def test_permute_mask_map_forward_backward(T, E, k, H, dtype, pdt, never, device
     probs = probs.to(pdt)
     gen = torch.Generator().manual_seed(T + 13)
     tokens = torch.randn(T, H, generator=gen).to(dtype)
-    exp_perm, exp_pp, exp_idx = O.permute_routing_map(tokens, rmap, probs)
+    # fused=True: the reference hook's dtype rule (one fp32 operand, one 16-bit one: both results 16-bit);
+    # fused=False: Megatron's own permute, every result in its operand's dtype.  Same kernels either way.
+    exp_perm, exp_pp, exp_idx = O.fused_permute_routing_map(tokens, rmap, probs)
+    plain_perm, plain_pp, _ = O.permute_routing_map(tokens, rmap, probs)
 
     tok_d = tokens.to(device).requires_grad_(True)
     probs_d = probs.to(device).requires_grad_(True)
+    perm_plain, pp_plain, sidx_plain = M.permute(tok_d, rmap.to(device), probs_d, fused=False)
+    assert perm_plain.dtype == dtype and pp_plain.dtype == pdt and torch.equal(sidx_plain.cpu(), exp_idx)
+    assert torch.equal(perm_plain.detach().cpu(), plain_perm) and torch.equal(pp_plain.detach().cpu(), plain_pp)
     for num_out in (None, exp_perm.size(0)):
         perm, pp, sidx = M.permute(tok_d, rmap.to(device), probs_d, num_out_tokens=num_out, fused=True)
         torch.cuda.synchronize()
         assert sidx.dtype == torch.int64 and torch.equal(sidx.cpu(), exp_idx)
-        assert torch.equal(perm.detach().cpu(), exp_perm)
-        assert torch.equal(pp.detach().cpu(), exp_pp)
+        assert perm.dtype == exp_perm.dtype and torch.equal(perm.detach().cpu(), exp_perm)
+        assert pp.dtype == exp_pp.dtype and torch.equal(pp.detach().cpu(), exp_pp)
 
     # backward: random cotangents for both differentiable outputs
-    g_rows = torch.randn(exp_perm.shape, generator=gen).to(dtype)
-    g_pp = torch.randn(exp_pp.shape, generator=gen).to(pdt)
+    g_rows = torch.randn(exp_perm.shape, generator=gen).to(exp_perm.dtype)
+    g_pp = torch.randn(exp_pp.shape, generator=gen).to(exp_pp.dtype)
     (perm * g_rows.to(device)).sum().backward(retain_graph=True)
     act_grad = tok_d.grad.clone()
     tok_d.grad = None
@@ -105,7 +112,8 @@ def test_unpermute_mask_map_forward_backward(T, E, k, H, dtype, pdt, never, with
     assert rel_l2(rows_d.grad, r64.grad) <= TOL[dtype]
     if with_probs:
         mask = rmap.double()
-        assert rel_l2(probs_d.grad.cpu().double() * mask, p64.grad * mask) <= TOL[dtype]
+        # the probabilities' gradient is rounded to their own dtype
+        assert rel_l2(probs_d.grad.cpu().double() * mask, p64.grad * mask) <= max(TOL[dtype], TOL[pdt])
         assert torch.count_nonzero(probs_d.grad.cpu().double() * (1 - mask)) == 0   # unset entries get no gradient
 
 
@@ -126,14 +134,14 @@ def test_drop_and_pad(T, E, k, cap, H, dtype, device):
     gen = torch.Generator().manual_seed(T + 41)
     tokens = torch.randn(T, H, generator=gen).to(dtype)
     n = E * cap
-    exp_perm, exp_pp, exp_idx = O.permute_routing_map(tokens, rmap, probs, num_out_tokens=n, drop_and_pad=True)
+    exp_perm, exp_pp, exp_idx = O.fused_permute_routing_map(tokens, rmap, probs, num_out_tokens=n, drop_and_pad=True)
     tok_d = tokens.to(device).requires_grad_(True)
     probs_d = probs.to(device).requires_grad_(True)
     perm, pp, sidx = M.permute(tok_d, rmap.to(device), probs_d, num_out_tokens=n, fused=True, drop_and_pad=True)
     torch.cuda.synchronize()
     assert torch.equal(sidx.cpu(), exp_idx)
     assert torch.equal(perm.detach().cpu(), exp_perm)
-    assert torch.equal(pp.detach().cpu(), exp_pp)
+    assert pp.dtype == exp_pp.dtype and torch.equal(pp.detach().cpu(), exp_pp)
 
     g_rows = torch.randn(exp_perm.shape, generator=gen).to(dtype)
     (perm * g_rows.to(device)).sum().backward()
@@ -213,3 +221,29 @@ def test_argument_checks(device):
         M.unpermute(torch.randn(8, 8, device=device), torch.zeros(8, dtype=torch.int64, device=device), tokens.shape)
     with pytest.raises(RuntimeError):
         M.permute(tokens.cpu(), rmap.cpu())
+
+
+def test_row_map_is_remembered_on_the_mask(device):
+    """unpermute reuses the row map permute computed as long as it gets the same mask tensor in the same state,
+    whatever happened to sorted_indices in between; a changed or different mask is sorted again."""
+    T, E, k, H = 256, 8, 2, 64
+    rmap, probs = make_map(T, E, k, 123)
+    rmap_d, probs_d = rmap.to(device), probs.to(device)
+    tokens = torch.randn(T, H, device=device).to(torch.bfloat16)
+    perm, _, sidx = M.permute(tokens, rmap_d, probs_d, num_out_tokens=T * k, fused=True)
+    assert M._recall_row_map(rmap_d, T * k, False) is not None
+    calls = []
+    real = M.routing_map_row_maps
+    M.routing_map_row_maps = lambda *a, **kw: (calls.append(1), real(*a, **kw))[1]
+    try:
+        out1 = M.unpermute(perm, sidx.clone(), tokens.shape, probs=probs_d, routing_map=rmap_d, fused=True)
+        assert not calls                                     # served from the remembered map
+        out2 = M.unpermute(perm, sidx, tokens.shape, probs=probs_d, routing_map=rmap_d.clone(), fused=True)
+        assert len(calls) == 1                               # another tensor object: sorted afresh
+        rmap_d.logical_or_(rmap_d)                           # in-place op: version counter moves on
+        assert M._recall_row_map(rmap_d, T * k, False) is None
+        out3 = M.unpermute(perm, sidx, tokens.shape, probs=probs_d, routing_map=rmap_d, fused=True)
+        assert len(calls) == 2
+    finally:
+        M.routing_map_row_maps = real
+    assert torch.equal(out1, out2) and torch.equal(out1, out3)

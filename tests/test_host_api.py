@@ -148,3 +148,75 @@ def test_fused_mlp_argument_checks():
         ops.gmm_swiglu(x, w1, torch.tensor([4, 4]))
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         ops.grouped_mlp(x, w1, torch.randn(2, 4, 16, dtype=torch.bfloat16), torch.tensor([4, 4]))
+
+
+def test_megatron_adapter_surface():
+    """``Ops`` is what Megatron's ``grouped_gemm_util.ops`` is replaced by
+    (mindspeed/core/fusions/grouped_matmul.py:5-21,35-50): same signature and defaults."""
+    from mindspeed_amd import fusions
+
+    sig = inspect.signature(fusions.Ops.gmm)
+    assert list(sig.parameters) == ["a", "b", "batch_sizes", "trans_b", "gemm_fusion", "original_weight"]
+    assert [sig.parameters[n].default for n in ("trans_b", "gemm_fusion", "original_weight")] == [False, False, None]
+    assert fusions.grouped_gemm_is_available() is True
+    fusions.assert_grouped_gemm_is_available()
+    assert fusions.get_device_capability() == (9, 0)
+    # mindspeed/core/fusions/fused_moe_permute.py:50-83
+    assert list(inspect.signature(fusions.permute).parameters) == [
+        "tokens", "routing_map", "probs", "num_out_tokens", "fused", "drop_and_pad"]
+    assert list(inspect.signature(fusions.unpermute).parameters) == [
+        "permuted_tokens", "sorted_indices", "restore_shape", "probs", "routing_map", "fused", "drop_and_pad"]
+    x = torch.randn(8, 16, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        fusions.Ops.gmm(x, torch.randn(2, 16, 4, dtype=torch.bfloat16), torch.tensor([4, 4]))
+
+
+def test_shapes_propagate_on_meta_tensors():
+    """Every op of the layer carries a fake (meta) kernel, so the Python surface runs on meta tensors, forward and
+    backward, without a device: ``torch.ops.mindspeed.npu_gmm`` yields ``(M, N)`` as the reference's Meta
+    registration does (mindspeed/op_builder/gmm_builder.py:101-106,141-146)."""
+    from mindspeed_amd import fusions
+    from mindspeed_amd.dispatcher import dispatch_mlp_combine
+    from mindspeed_amd.ops import moe_permute_mask_map as M
+
+    def meta(*shape, dtype=torch.bfloat16, grad=False):
+        return torch.empty(*shape, dtype=dtype, device="meta", requires_grad=grad)
+
+    T, H, E, K, F = 64, 32, 4, 2, 48
+    x, w = meta(T * K, H, grad=True), meta(E, H, 2 * F, grad=True)
+    gl = meta(E, dtype=torch.int64)
+    for y in (torch.ops.mindspeed.npu_gmm(None, x, w, group_list=gl),
+              torch.ops.mindspeed.npu_gmm(None, x, w, group_list=[32, 64, 96, 128]),
+              torch.ops.mindspeed.npu_gmm_v2(None, x, w, group_list=gl),
+              ops.npu_gmm(x, w, group_list=gl), fusions.Ops.gmm(x, w, gl)):
+        assert y.device.type == "meta" and y.shape == (T * K, 2 * F) and y.dtype == torch.bfloat16
+    y.sum().backward()
+    assert x.grad.shape == x.shape and w.grad.shape == w.shape
+    assert fusions.Ops.gmm(x, meta(E, 2 * F, H), gl, trans_b=True).shape == (T * K, 2 * F)
+    dw = ops.npu_gmm(x.detach().t(), meta(T * K, 24), group_list=gl, group_type=2)
+    assert dw.shape == (E, H, 24)
+
+    tokens, idx = meta(T, H, grad=True), meta(T, K, dtype=torch.int64)
+    permuted, row_map = ops.npu_moe_token_permute(tokens, idx)
+    assert permuted.shape == (T * K, H) and row_map.shape == (T * K,) and row_map.dtype == torch.int32
+    assert ops.npu_moe_token_permute(tokens, idx, num_out_tokens=100)[0].shape == (100, H)
+    probs = meta(T, K, grad=True)
+    out = ops.npu_moe_token_unpermute(permuted, row_map, probs)
+    assert out.shape == (T, H)
+    out.sum().backward()
+    assert tokens.grad.shape == (T, H) and probs.grad.shape == (T, K)
+
+    w1, w2 = meta(E, H, 2 * F, grad=True), meta(E, F, H, grad=True)
+    out = dispatch_mlp_combine(tokens, idx, probs, (w1, w2))
+    assert out.shape == (T, H)
+    out.sum().backward()
+    assert w1.grad.shape == w1.shape and w2.grad.shape == w2.shape
+
+    rmap, mprobs = meta(T, E, dtype=torch.bool), meta(T, E, dtype=torch.float32, grad=True)
+    perm, pp, sidx = M.permute(tokens, rmap, mprobs, num_out_tokens=T * K, fused=True)
+    assert perm.shape == (T * K, H) and pp.shape == (T * K,) and sidx.dtype == torch.int64
+    assert perm.dtype == torch.bfloat16 and pp.dtype == torch.bfloat16       # the fused hook's dtype rule
+    back = M.unpermute(perm, sidx, tokens.shape, probs=mprobs, routing_map=rmap, fused=True)
+    assert back.shape == (T, H)
+    back.sum().backward()
+    assert mprobs.grad.shape == (T, E)

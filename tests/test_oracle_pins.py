@@ -372,3 +372,29 @@ def test_row_reference_agrees_with_oracle_autograd():
         assert torch.allclose(u, dw1[e][ks][:, cfg["F"] + fs], rtol=1e-5, atol=1e-5)
         assert torch.allclose(d2, dw2[e][fs][:, hs], rtol=1e-5, atol=1e-5)
     assert ref.counts[4] == 0 and torch.count_nonzero(dw1[4]) == 0
+
+
+def test_fused_permute_dtype_rule():
+    """Result dtypes of the reference's fused permute hook (mindspeed/core/fusions/fused_moe_permute.py:17-47,58-63),
+    typed by hand from the rule: promote both to fp32 iff exactly one is fp32, then cast both to the other one's
+    dtype.  Values are those of the plain permutation (a gather moves bits) rounded to the result dtype."""
+    f32, b16, h16 = torch.float32, torch.bfloat16, torch.float16
+    table = {
+        (b16, b16): (b16, b16), (b16, f32): (b16, b16), (f32, b16): (b16, b16), (f32, f32): (f32, f32),
+        (h16, f32): (h16, h16), (f32, h16): (h16, h16), (h16, h16): (h16, h16),
+        (b16, h16): (b16, h16),      # two different 16-bit types: nothing is promoted, nothing is cast
+    }
+    gen = torch.Generator().manual_seed(4)
+    T, E, H = 12, 5, 6
+    rmap = torch.rand(T, E, generator=gen) < 0.4
+    base_t = torch.randn(T, H, generator=gen)
+    base_p = torch.rand(T, E, generator=gen)
+    for (tdt, pdt), (want_t, want_p) in table.items():
+        tokens, probs = base_t.to(tdt), base_p.to(pdt)
+        perm, pp, sidx = O.fused_permute_routing_map(tokens, rmap, probs)
+        assert (perm.dtype, pp.dtype) == (want_t, want_p), (tdt, pdt)
+        plain_t, plain_p, plain_idx = O.permute_routing_map(tokens, rmap, probs)
+        assert torch.equal(sidx, plain_idx)
+        assert torch.equal(perm, plain_t.to(want_t)) and torch.equal(pp, plain_p.to(want_p))
+    perm, pp, _ = O.fused_permute_routing_map(base_t.to(b16), rmap, None)
+    assert perm.dtype == b16 and pp is None
