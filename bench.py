@@ -28,12 +28,39 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}   # dense, published
 
-# HBM bytes per launch of the dominant kernel (forward grouped matmul, fc1/fc2 average) from rocprofv3
-# FETCH_SIZE + WRITE_SIZE, scaled by what the same counters read for the plain copy kernel of known size
-# (profiles/moe_layer_mixtral_hbm_traffic.txt).  None where it has not been measured.
-TRAFFIC_BYTES_PER_LAUNCH = {"mixtral": 5227968600}
-
 from mindspeed_amd.workloads import WORKLOADS, make_inputs, make_routing  # noqa: E402
+
+# HBM bytes per launch of each grouped-matmul flavour (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by what the same
+# counters read for the plain copy kernel of known size), written by `python -m mindspeed_amd.profile_tools traffic`
+# together with the hash of the kernel sources they were measured on.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gmm_hbm_traffic.json")
+
+GEMM_KERNEL_NAMES = {
+    "gmm_fwd": "gmm16_fast_kernel<bf16, A reduction-contiguous, B column-contiguous> (forward grouped matmul; one "
+               "launch each for fc1 and fc2, averaged)",
+    "gmm_dx": "gmm16_fast_kernel<bf16, A reduction-contiguous, B reduction-contiguous> (dX grouped matmul on the "
+              "transposed weight view; one launch each for fc1 and fc2, averaged)",
+    "gmm_dw": "gmm16_fast_kernel<bf16, A row-contiguous, B column-contiguous> (dW grouped matmul, split on the "
+              "reduction dim; one launch each for fc1 and fc2, averaged)",
+    "gmm_fwd_swiglu": "gmm16_fast_kernel<bf16, A reduction-contiguous, B column-contiguous, SwiGLU epilogue> (fc1 "
+                      "forward grouped matmul, one launch per step)",
+    "gmm_dx_swiglu": "gmm16_fast_kernel<bf16, A, B reduction-contiguous, SwiGLU-backward epilogue> (fc2 dX grouped "
+                     "matmul, one launch per step)",
+}
+
+
+def measured_traffic(workload, kernel):
+    """Bytes per launch from the tracked profile, or None when there is none for this workload / kernel or the kernel
+    sources have changed since it was taken."""
+    from mindspeed_amd.build import source_hash
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            data = json.load(fh)
+    except (OSError, ValueError):
+        return None
+    if data.get("build") != source_hash():
+        return None
+    return data.get("bytes_per_launch", {}).get(workload, {}).get(kernel)
 
 
 def _cpu_layer_once(cfg, sample):
@@ -54,9 +81,21 @@ def _cpu_layer_once(cfg, sample):
     return time.perf_counter() - t0
 
 
-def cpu_baseline(cfg, budget_s=15.0):
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for line in fh:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(cfg, budget_s=12.0):
     """The CPU oracle (torch restatement of the reference's pure-PyTorch path) timed on this host, fp32,
-    forward + backward, on a token sample sized (from a short probe run) to about budget_s of CPU work."""
+    forward + backward, on a token sample sized (from a short probe run) to about budget_s of CPU work; then the same
+    on one thread with a smaller sample."""
     threads = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
     T = cfg["T"]
@@ -65,9 +104,17 @@ def cpu_baseline(cfg, budget_s=15.0):
     sample = int(min(T, max(probe, probe * budget_s / max(t_probe, 1e-3))))
     sample = max(64, (sample // 64) * 64) if sample >= 64 else sample
     dt = _cpu_layer_once(cfg, sample) if sample != probe else _cpu_layer_once(cfg, probe)
+    torch.set_num_threads(1)
+    one = min(sample, 64)
+    dt1 = _cpu_layer_once(cfg, one)
+    torch.set_num_threads(threads)
     return {"value": round(sample / dt, 2), "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": f"{sample} of {T} tokens, same layer shape, fp32, one forward+backward "
-                      f"({dt:.1f} s) with torch {torch.__version__} on {threads} threads"}
+            "sample": f"{sample} of {T} tokens (extrapolated: every expert still reads its whole fp32 weights for that "
+                      f"few rows, which is pessimistic for the CPU), same layer shape, fp32, one forward+backward "
+                      f"({dt:.1f} s) with torch {torch.__version__} on {threads} threads",
+            "single_thread": {"value": round(one / dt1, 2), "unit": "tokens/s", "cores": 1,
+                              "sample": f"{one} tokens, one forward+backward ({dt1:.1f} s)"},
+            "cpu_model": _cpu_model(), "host_cores": os.cpu_count()}
 
 
 def measure_routing_map_mode(cfg, device, x, idx, p, iters=20, warmup=5):
@@ -122,6 +169,57 @@ def measure_routing_map_mode(cfg, device, x, idx, p, iters=20, warmup=5):
     }
 
 
+def run_layer(cfg, device, steps, warmup, fuse_activation=False, per_kernel=True):
+    """`warmup` untimed steps, exactly `steps` timed ones between two synchronisations, then (per_kernel) the same
+    steps again with every op bracketed by two events on its launch stream.  Returns (ms per step, ms per step with
+    the event brackets or None, per-kernel table or None, the inputs)."""
+    from mindspeed_amd import flop_counter
+    from mindspeed_amd.dispatcher import dispatch_mlp_combine
+
+    x, p, idx, w1, w2, gy = make_inputs(cfg, device)
+    leaves = [t.requires_grad_(True) for t in (x, p, w1, w2)]
+
+    def step():
+        out = dispatch_mlp_combine(leaves[0], idx, leaves[1], (leaves[2], leaves[3]), fuse_activation=fuse_activation)
+        return torch.autograd.grad(out, leaves, gy)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    # timed region: exactly `steps` steps, nothing else on the stream
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+    if not per_kernel:
+        return ms_per_step, None, None, (x, p, idx)
+
+    with flop_counter.record(timing=True) as rec:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        ms_events = (time.perf_counter() - t0) * 1e3 / steps
+    peak = MFMA_PEAK_TFLOPS[cfg["dtype"]]
+    kernels = {}
+    for name, s in rec.summary().items():
+        avg_ms = s["ms"] / s["calls"]
+        work = s["work"] / s["calls"]
+        entry = {"calls_per_step": s["calls"] / steps, "avg_ms": round(avg_ms, 5),
+                 "ms_per_step": round(s["ms"] / steps, 5)}
+        if s["unit"] == "flop":
+            entry["tflops"] = round(work / (avg_ms * 1e-3) / 1e12, 2)
+            entry["flop_per_launch"] = work
+            entry["frac_of_mfma_peak"] = round(entry["tflops"] / peak, 4)
+        else:
+            entry["gbs"] = round(work / (avg_ms * 1e-3) / 1e9, 1)
+            entry["bytes_per_launch"] = work
+            entry["frac_of_hbm_peak"] = round(entry["gbs"] / HBM_PEAK_GBS, 4)
+        kernels[name] = entry
+    return ms_per_step, ms_events, kernels, (x, p, idx)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -129,6 +227,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="mixtral", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="only the timed steps and the per-kernel table (no other workloads, no permute-family or "
+                         "routing-map sections)")
     ap.add_argument("--fuse-activation", action="store_true",
                     help="run the expert MLP with SwiGLU fused into the neighbouring grouped matmuls "
                          "(default: the reference's op sequence, one kernel per op)")
@@ -142,41 +243,14 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a HIP device")
 
-    from mindspeed_amd import flop_counter
-    from mindspeed_amd.dispatcher import dispatch_mlp_combine
-
     cfg = WORKLOADS[args.workload]
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
-    x, p, idx, w1, w2, gy = make_inputs(cfg, device)
-    leaves = [t.requires_grad_(True) for t in (x, p, w1, w2)]
-
-    def step():
-        out = dispatch_mlp_combine(leaves[0], idx, leaves[1], (leaves[2], leaves[3]),
-                                   fuse_activation=args.fuse_activation)
-        return torch.autograd.grad(out, leaves, gy)
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    # timed region: exactly K steps, nothing else on the stream
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
+    ms_per_step, ms_per_step_events, kernels, (x, p, idx) = run_layer(
+        cfg, device, args.steps, args.warmup, args.fuse_activation)
     tokens_per_s = cfg["T"] / (ms_per_step / 1e3)
 
-    # the same K steps again with every op bracketed by two events on its launch stream: per-kernel times
-    with flop_counter.record(timing=True) as rec:
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        ms_per_step_events = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    # what an empty bracket reads: the per-op times below include this much that is not the kernel
+    # what an empty bracket reads: the per-op times include this much that is not the kernel
     stream = torch.cuda.current_stream(device)
     pairs = []
     for _ in range(50):
@@ -187,41 +261,17 @@ def main():
     torch.cuda.synchronize()
     empty_bracket_ms = sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
 
-    kernels = {}
-    for name, s in rec.summary().items():
-        avg_ms = s["ms"] / s["calls"]
-        work = s["work"] / s["calls"]
-        entry = {"calls_per_step": s["calls"] / args.steps, "avg_ms": round(avg_ms, 5)}
-        if s["unit"] == "flop":
-            entry["tflops"] = round(work / (avg_ms * 1e-3) / 1e12, 2)
-            entry["flop_per_launch"] = work
-        else:
-            entry["gbs"] = round(work / (avg_ms * 1e-3) / 1e9, 1)
-            entry["bytes_per_launch"] = work
-        kernels[name] = entry
-
+    # dominant kernel: the grouped-matmul flavour with the largest share of the step
     peak = MFMA_PEAK_TFLOPS[cfg["dtype"]]
-    # dominant kernel: the largest launch of the step, the first grouped matmul of the forward pass (fc1), which
-    # also carries the SwiGLU epilogue when the layer runs fused (the activation math is not in the flop count)
-    fused = "gmm_fwd_swiglu" in kernels
-    dom = kernels["gmm_fwd_swiglu" if fused else "gmm_fwd"]
-    if cfg["dtype"] != "bf16":
-        kname = "gmm32_kernel (forward grouped matmul, fp32)"
-    elif fused:
-        kname = ("gmm16_fast_kernel<bf16, A reduction-contiguous, B column-contiguous, SwiGLU epilogue> "
-                 "(fc1 forward grouped matmul, one launch per step)")
-    else:
-        kname = ("gmm16_fast_kernel<bf16, A reduction-contiguous, B column-contiguous> (forward grouped matmul; "
-                 "one launch each for fc1 and fc2, averaged)")
-    roofline = {"bound": "mfma", "kernel": kname,
-                "achieved": dom["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": round(dom["tflops"] / peak, 4),
-                "traffic": None if fused else TRAFFIC_BYTES_PER_LAUNCH.get(args.workload)}
-    for name, e in kernels.items():
-        if "tflops" in e:
-            e["frac_of_mfma_peak"] = round(e["tflops"] / peak, 4)
-    for name, e in kernels.items():
-        if "gbs" in e:
-            e["frac_of_hbm_peak"] = round(e["gbs"] / HBM_PEAK_GBS, 4)
+    gemms = {k: v for k, v in kernels.items() if "tflops" in v}
+    dom_name = max(gemms, key=lambda k: gemms[k]["ms_per_step"])
+    dom = gemms[dom_name]
+    kname = GEMM_KERNEL_NAMES.get(dom_name, dom_name) if cfg["dtype"] == "bf16" else \
+        f"gmm32_kernel ({dom_name}, fp32 inputs)"
+    roofline = {"bound": "mfma", "kernel": kname, "kernel_key": dom_name,
+                "share_of_step": round(dom["ms_per_step"] / sum(v["ms_per_step"] for v in kernels.values()), 4),
+                "achieved": dom["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": dom["frac_of_mfma_peak"],
+                "traffic": measured_traffic(args.workload, dom_name)}
 
     result = {
         "metric": "MoE layer fwd+bwd tokens/s at 1 GPU",
@@ -239,12 +289,12 @@ def main():
         "data": "synthetic",
         "config": {"workload": cfg["desc"], "tokens": cfg["T"], "hidden": cfg["H"], "experts": cfg["E"],
                    "topk": cfg["K"], "ffn": cfg["F"], "fused_activation": bool(args.fuse_activation),
-                   "gemm_tflop_per_step": round(18.0 * cfg["T"] * cfg["K"]
-                                                                                  * cfg["H"] * cfg["F"] / 1e12, 3)},
+                   "gemm_tflop_per_step": round(18.0 * cfg["T"] * cfg["K"] * cfg["H"] * cfg["F"] / 1e12, 3)},
         "roofline": roofline,
         "kernels": kernels,
-        "kernels_note": "single launches inside the layer step, each between two events on its stream; an empty "
-                        f"bracket reads {empty_bracket_ms * 1e3:.1f} us on this box",
+        "kernels_note": "single launches inside the layer step, each between two events on its stream (the two "
+                        "weight-gradient products then run after, not beside, the dX products); an empty bracket "
+                        f"reads {empty_bracket_ms * 1e3:.1f} us on this box",
     }
     if args.copy_calibration:
         from mindspeed_amd import _lib
@@ -256,15 +306,40 @@ def main():
             _lib.check(lib.ms_copy_bytes(_lib.stream_ptr(device), _lib.ptr(src), _lib.ptr(dst), n), "ms_copy_bytes")
         torch.cuda.synchronize()
         result["copy_calibration_bytes"] = n
-    result["routing_map_mode"] = measure_routing_map_mode(cfg, device, x.detach(), idx, p.detach())
-    # The permute / unpermute family by itself at this workload's shape: back-to-back launches through the C ABI
-    # on resident buffers (the per-op figures under "kernels" are single launches inside the layer step, bracketed
-    # by events, i.e. with the launch gaps on either side).  Not part of `value`.
-    from mindspeed_amd.permute_microbench import measure as measure_permute_family
-    result["permute_family"] = {
-        "note": "back-to-back launches through the C ABI, event-timed over 200 launches per op; "
-                "algorithmic bytes over the average, against the 8 TB/s HBM peak",
-        **measure_permute_family(cfg["T"], cfg["H"], cfg["E"], cfg["K"], torch.bfloat16, device=device)}
+    if not args.no_extras:
+        result["routing_map_mode"] = measure_routing_map_mode(cfg, device, x.detach(), idx, p.detach())
+        # The permute / unpermute family by itself at this workload's shape: back-to-back launches through the C ABI
+        # (the per-op figures under "kernels" are single launches inside the layer step, whose operands were last
+        # touched hundreds of megabytes of traffic earlier).  "warm": one set of buffers, resident in the 256 MB
+        # last-level cache at this size; "cold": launches rotate through enough buffer sets to exceed that cache
+        # six times, so every launch streams from HBM.  Not part of `value`.
+        from mindspeed_amd.permute_microbench import measure as measure_permute_family, sets_for_cold
+        shape = (cfg["T"], cfg["H"], cfg["E"], cfg["K"], torch.bfloat16)
+        cold_sets = sets_for_cold(cfg["T"], cfg["H"], cfg["K"])
+        warm = measure_permute_family(*shape, device=device)
+        cold = measure_permute_family(*shape, device=device, sets=cold_sets)
+        for table in (warm, cold):
+            for r in table.values():
+                r["frac_of_copy"] = round(r["gbs"] / table["copy"]["gbs"], 3)
+        result["permute_family"] = {
+            "note": "back-to-back launches through the C ABI, event-timed over 200 launches per op; algorithmic bytes "
+                    "over the average, against the 8 TB/s HBM peak and against the plain copy kernel in the same mode",
+            "cold_buffer_sets": cold_sets, "warm": warm, "cold": cold}
+        # the other two bf16 workloads, forward+backward, 10 steps each after their own warm-up
+        if args.workload == "mixtral":
+            others = {}
+            del x, p, idx
+            torch.cuda.empty_cache()
+            for name in ("deepseek", "qwen"):
+                ocfg = WORKLOADS[name]
+                ms, _, ok, _ = run_layer(ocfg, device, steps=10, warmup=10)
+                others[name] = {"workload": ocfg["desc"], "ms_per_step": round(ms, 4),
+                                "tokens_per_s": round(ocfg["T"] / (ms / 1e3), 1),
+                                "gemm_tflops": {k: ok[k]["tflops"] for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok},
+                                "gemm_frac_of_mfma_peak": {k: ok[k]["frac_of_mfma_peak"]
+                                                           for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok}}
+                torch.cuda.empty_cache()
+            result["other_workloads"] = others
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(result))

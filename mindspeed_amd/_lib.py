@@ -12,7 +12,8 @@ import threading
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmindspeed_amd.so")
+# MINDSPEED_AMD_LIB names another build of the same library (to compare two builds on one machine)
+LIB_PATH = os.environ.get("MINDSPEED_AMD_LIB") or os.path.join(_HERE, "libmindspeed_amd.so")
 
 MS_BF16, MS_FP16, MS_FP32 = 0, 1, 2
 MS_INT32, MS_INT64 = 0, 1

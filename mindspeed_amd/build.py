@@ -37,9 +37,25 @@ def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
+def source_hash() -> str:
+    """First 16 hex digits of the SHA-256 over the kernel sources (csrc/*.hip, csrc/*.h, the C-ABI header) in name
+    order: names the build that measured figures (profiles/*.json) belong to."""
+    import hashlib
+
+    h = hashlib.sha256()
+    files = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hip", ".h")))
+    files.append(os.path.join(HERE, "..", "include", "mindspeed_amd.h"))
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
 def _compile(src: str, force: bool) -> str:
     obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
-    deps = [src, os.path.join(CSRC, "common.h"), os.path.join(HERE, "..", "include", "mindspeed_amd.h")]
+    deps = [src, os.path.join(HERE, "..", "include", "mindspeed_amd.h")]
+    deps += [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) > os.path.getmtime(d) for d in deps):
         return obj
     cmd = [_hipcc(), *HIPCC_FLAGS, "-c", src, "-o", obj]

@@ -1,0 +1,259 @@
+"""Measurement helpers behind the figures under ``profiles/``.
+
+    python -m mindspeed_amd.profile_tools traffic --fetch F.csv --write W.csv [--workload mixtral] [--out FILE.json]
+    python -m mindspeed_amd.profile_tools counters CSV [CSV ...]
+    python -m mindspeed_amd.profile_tools power [--seconds 4] [--modes fwd1,dx1,dw1,library] [--data randn,zeros]
+
+``traffic`` reads the ``*_counter_collection.csv`` files of two ``rocprofv3 --pmc`` runs of ``bench.py`` (one with
+FETCH_SIZE, one with WRITE_SIZE; both with ``--copy-calibration MIB`` so that the plain copy kernel of known size is
+among the dispatches), scales the counters by what they read for that copy, prints HBM bytes per dispatch for every
+kernel of the library and, with ``--out``, records the grouped-matmul figures together with the hash of the kernel
+sources they belong to (``bench.py`` reports them as ``roofline.traffic`` as long as that hash is unchanged).
+
+``counters`` prints per-kernel averages of whatever counters the given files hold.
+
+``power`` runs one grouped-matmul launch of the Mixtral-shape expert MLP back to back for a few seconds per
+(product, operand values) pair while a thread samples the board's power draw and shader clock from the amdgpu
+hwmon / sysfs files (read-only), and prints rate, power and clock side by side.
+"""
+from __future__ import annotations
+
+import argparse
+import collections
+import csv
+import glob
+import json
+import os
+import re
+import sys
+import threading
+import time
+
+GEMM_KEYS = {  # template arguments <dtype, A reduction-contiguous, B reduction-contiguous, output mode>
+    "gmm16_fast_kernel<0, true, false, 0>": "gmm_fwd",
+    "gmm16_fast_kernel<0, true, true, 0>": "gmm_dx",
+    "gmm16_fast_kernel<0, false, false, 0>": "gmm_dw",
+    "gmm16_fast_kernel<0, true, false, 3>": "gmm_fwd_swiglu",
+    "gmm16_fast_kernel<0, true, true, 4>": "gmm_dx_swiglu",
+}
+
+
+def short_name(name: str) -> str:
+    name = name.replace("void ", "").replace("ms::(anonymous namespace)::", "")
+    name = re.sub(r"\(.*$", "", name)
+    return name.replace("(ms::OutMode)", "").replace("(int)", "")
+
+
+def read_counter(path: str, counter: str):
+    """kernel -> list of per-dispatch values of `counter`."""
+    per_kernel = collections.defaultdict(list)
+    with open(path, newline="") as fh:
+        for row in csv.DictReader(fh):
+            if row["Counter_Name"] == counter:
+                per_kernel[short_name(row["Kernel_Name"])].append(float(row["Counter_Value"]))
+    return per_kernel
+
+
+def calibration(per_kernel, known_kib: float):
+    """Scale factor of a byte counter from the copy kernel's largest dispatches (a transfer of `known_kib` KiB)."""
+    copies = [v for k, vals in per_kernel.items() if "copy_bytes_kernel" in k for v in vals]
+    if not copies:
+        raise SystemExit("no copy_bytes_kernel dispatches in the counter file: run bench.py with --copy-calibration MIB")
+    big = [v for v in copies if v >= 0.9 * max(copies)]
+    return known_kib / (sum(big) / len(big)), sum(big) / len(big), len(big)
+
+
+def cmd_traffic(args):
+    from .build import source_hash
+
+    fetch = read_counter(args.fetch, "FETCH_SIZE")
+    write = read_counter(args.write, "WRITE_SIZE")
+    known_kib = args.copy_mib * 1024.0
+    f_scale, f_read, f_n = calibration(fetch, known_kib)
+    w_scale, w_read, w_n = calibration(write, known_kib)
+    print(f"calibration: {f_n} copy_bytes_kernel dispatches over {args.copy_mib} MiB read FETCH_SIZE = {f_read:.0f}, "
+          f"WRITE_SIZE = {w_read:.0f} (KiB moved each way: {known_kib:.0f})")
+    print(f"  -> scale factors: FETCH_SIZE x {f_scale:.3f}, WRITE_SIZE x {w_scale:.3f}\n")
+    print(f"{'kernel':84s} {'disp':>5s} {'fetch_MB':>10s} {'write_MB':>10s} {'total_MB':>10s}")
+    record = {}
+    for kernel in fetch:
+        if "ms::" not in kernel and "gmm" not in kernel and "kernel" not in kernel:
+            continue
+        f = fetch[kernel]
+        w = write.get(kernel, [])
+        if not w:
+            continue
+        f_mb = sum(f) / len(f) * f_scale * 1024 / 1e6
+        w_mb = sum(w) / len(w) * w_scale * 1024 / 1e6
+        print(f"{kernel[:84]:84s} {len(f):5d} {f_mb:10.1f} {w_mb:10.1f} {f_mb + w_mb:10.1f}")
+        for pattern, key in GEMM_KEYS.items():
+            if pattern in kernel:
+                record[key] = int(round((f_mb + w_mb) * 1e6))
+    if args.out:
+        data = {}
+        if os.path.exists(args.out):
+            with open(args.out) as fh:
+                data = json.load(fh)
+        build = source_hash()
+        if data.get("build") != build:
+            data = {"build": build, "unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by the copy "
+                                            "kernel's reading; launches of fc1 and fc2 averaged)", "bytes_per_launch": {}}
+        data["bytes_per_launch"][args.workload] = record
+        with open(args.out, "w") as fh:
+            json.dump(data, fh, indent=1, sort_keys=True)
+            fh.write("\n")
+        print(f"\nrecorded {record} for build {build} in {args.out}")
+
+
+def cmd_counters(args):
+    for path in args.files:
+        agg = collections.defaultdict(lambda: collections.defaultdict(list))
+        with open(path, newline="") as fh:
+            for row in csv.DictReader(fh):
+                agg[short_name(row["Kernel_Name"])][row["Counter_Name"]].append(float(row["Counter_Value"]))
+        print(f"# {os.path.basename(path)}")
+        for kernel, counters in agg.items():
+            for counter, vals in counters.items():
+                print(f"{kernel[:90]:90s} {counter:28s} dispatches {len(vals):5d}  avg {sum(vals) / len(vals):16.1f}")
+
+
+# ---- power / clock ---------------------------------------------------------------------------------------------
+def _hwmon_dirs():
+    return sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))
+
+
+def _read(path):
+    try:
+        with open(path) as fh:
+            return fh.read().strip()
+    except OSError:
+        return None
+
+
+def sample_board():
+    """(watts, shader MHz) of the first GPU, from the amdgpu hwmon and pp_dpm_sclk files; None where unreadable."""
+    watts = mhz = None
+    for h in _hwmon_dirs():
+        for name in ("power1_input", "power1_average"):
+            v = _read(os.path.join(h, name))
+            if v is not None:
+                watts = int(v) / 1e6
+                break
+        sclk = _read(os.path.join(os.path.dirname(os.path.dirname(h)), "pp_dpm_sclk"))
+        if sclk:
+            for line in sclk.splitlines():
+                if "*" in line:
+                    found = re.search(r"(\d+)\s*Mhz", line, re.I)
+                    if found:
+                        mhz = int(found.group(1))
+        if watts is not None:
+            break
+    return watts, mhz
+
+
+def cmd_power(args):
+    import torch
+
+    from .ops.gmm import gmm_raw
+
+    if not torch.cuda.is_available():
+        raise SystemExit("needs a HIP device")
+    dev = torch.device("cuda", 0)
+    T, H, F, E = 8192, 4096, 14336, 8
+    bf = torch.bfloat16
+    gen = torch.Generator(device=dev).manual_seed(0)
+    counts = torch.full((E,), T // E, dtype=torch.int64, device=dev)
+    cap = None
+    for h in _hwmon_dirs():
+        v = _read(os.path.join(h, "power1_cap"))
+        if v is not None:
+            cap = int(v) / 1e6
+    idle = sample_board()
+    print(f"Mixtral-shape fc1 products, {T} rows in {E} equal groups, hidden {H}, 2*ffn {2 * F}, bf16; "
+          f"{args.seconds:.0f} s of back-to-back launches per line")
+    print(f"board power cap {cap} W; idle reading {idle[0]} W at {idle[1]} MHz")
+    print(f"{'product':10s} {'operands':8s} {'ms':>8s} {'TFLOP/s':>8s} {'frac':>6s} {'W(avg)':>8s} {'W(max)':>8s} {'MHz(avg)':>9s}")
+
+    def operand(data, *shape):
+        if data == "zeros":
+            return torch.zeros(*shape, device=dev, dtype=bf)
+        if data == "ones":
+            return torch.ones(*shape, device=dev, dtype=bf)
+        if data == "small":
+            return torch.randint(-2, 3, shape, generator=gen, device=dev).to(bf)
+        return torch.randn(*shape, generator=gen, device=dev).to(bf)
+
+    flops = 2 * T * H * 2 * F
+    for mode in args.modes.split(","):
+        for data in args.data.split(","):
+            if mode == "fwd1":
+                x, w = operand(data, T, H), operand(data, E, H, 2 * F)
+                fn = lambda: gmm_raw(x, w, counts, 0, 1)            # noqa: E731
+            elif mode == "dx1":
+                dy, w = operand(data, T, 2 * F), operand(data, E, H, 2 * F)
+                fn = lambda: gmm_raw(dy, w.transpose(1, 2), counts, 0, 1)   # noqa: E731
+            elif mode == "dw1":
+                x, dy = operand(data, T, H), operand(data, T, 2 * F)
+                fn = lambda: gmm_raw(x.t(), dy, counts, 2, 1)      # noqa: E731
+            elif mode == "library":   # torch.bmm (the vendor library) on the same shape as E dense products, for orientation
+                x, w = operand(data, E, T // E, H), operand(data, E, H, 2 * F)
+                fn = lambda: torch.bmm(x, w)                       # noqa: E731
+            else:
+                raise SystemExit(f"unknown mode {mode}")
+            for _ in range(30):
+                fn()
+            torch.cuda.synchronize()
+            samples = []
+            stop = threading.Event()
+
+            def sampler():
+                while not stop.is_set():
+                    samples.append(sample_board())
+                    time.sleep(0.2)
+            thread = threading.Thread(target=sampler)
+            thread.start()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0, n = time.time(), 0
+            e0.record()
+            while time.time() - t0 < args.seconds:
+                for _ in range(50):
+                    fn()
+                torch.cuda.synchronize()
+                n += 50
+            e1.record()
+            torch.cuda.synchronize()
+            stop.set()
+            thread.join()
+            ms = e0.elapsed_time(e1) / n
+            steady = samples[len(samples) // 4:] or samples       # drop the ramp at the start
+            watts = [s[0] for s in steady if s[0] is not None]
+            mhz = [s[1] for s in steady if s[1] is not None]
+            tf = flops / ms / 1e9
+            print(f"{mode:10s} {data:8s} {ms:8.4f} {tf:8.0f} {tf / 2500:6.3f} "
+                  f"{(sum(watts) / len(watts)) if watts else float('nan'):8.0f} {max(watts) if watts else float('nan'):8.0f} "
+                  f"{(sum(mhz) / len(mhz)) if mhz else float('nan'):9.0f}", flush=True)
+            del fn
+            time.sleep(1.0)
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    sub = ap.add_subparsers(dest="cmd", required=True)
+    t = sub.add_parser("traffic")
+    t.add_argument("--fetch", required=True)
+    t.add_argument("--write", required=True)
+    t.add_argument("--workload", default="mixtral")
+    t.add_argument("--copy-mib", type=int, default=1024)
+    t.add_argument("--out", default="")
+    c = sub.add_parser("counters")
+    c.add_argument("files", nargs="+")
+    w = sub.add_parser("power")
+    w.add_argument("--seconds", type=float, default=4.0)
+    w.add_argument("--modes", default="fwd1,dx1,dw1,library")
+    w.add_argument("--data", default="randn,small,zeros")
+    args = ap.parse_args()
+    {"traffic": cmd_traffic, "counters": cmd_counters, "power": cmd_power}[args.cmd](args)
+
+
+if __name__ == "__main__":
+    sys.exit(main())
