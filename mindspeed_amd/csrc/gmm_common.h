@@ -65,7 +65,7 @@ struct TileCoord {
 
 // Map this workgroup to its tile.  Workgroup b runs on XCD b % 8 (round-robin dispatch) and takes slot
 // b / 8 of that XCD's slot sequence.  Every XCD walks the groups in the same order and owns one contiguous
-// eighth of each group's tiles (row-tile-fastest inside a column panel), so concurrently running
+// eighth of each group's tiles (in the blocked order below), so concurrently running
 // workgroups of an XCD share operand panels in that XCD's L2, and every XCD gets an equal part of every
 // group however unequal the groups are.
 __device__ __forceinline__ TileCoord locate_tile(const TileTable *table) {
@@ -82,8 +82,22 @@ __device__ __forceinline__ TileCoord locate_tile(const TileTable *table) {
     tc.e = table->entries[lo];
     const int r = xcd * tc.e.share + (slot - tc.e.tile_begin);
     if (r >= tc.e.num_tiles) return tc;
-    tc.col_tile = r / tc.e.num_row_tiles;
-    tc.row_tile = r - tc.col_tile * tc.e.num_row_tiles;
+    // Tile order inside a group: column panels in sets of 8, row tiles in sets of 4, row-tile-fastest inside such a
+    // 4 x 8 block.  The 32 compute units of an XCD then work on one block at a time and fetch 4 + 8 operand panels
+    // for 32 tiles; with many row tiles (the weight gradient: hidden / 256 of them) plain row-tile-fastest order
+    // would have them on 16 x 2 tiles and fetch 18.  Up to 4 row tiles per group the two orders are the same.
+    {
+        const int R = tc.e.num_row_tiles, C = tc.e.num_tiles / R;
+        const int cg = r / (8 * R);
+        const int rem = r - cg * 8 * R;
+        const int wc = C - 8 * cg < 8 ? C - 8 * cg : 8;        // column panels in this set
+        const int rb = rem / (4 * wc);
+        const int rem2 = rem - rb * 4 * wc;
+        const int hr = R - 4 * rb < 4 ? R - 4 * rb : 4;        // row tiles in this block
+        const int lc = rem2 / hr;
+        tc.col_tile = 8 * cg + lc;
+        tc.row_tile = 4 * rb + (rem2 - lc * hr);
+    }
     tc.tile_rows = (tc.e.tail_rows != 0 && tc.row_tile == tc.e.num_row_tiles - 1) ? tc.e.tail_rows : tc.e.tile_rows;
     tc.valid = true;
     return tc;
