@@ -16,6 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libmindspeed_amd.so")
+TRACE_LIB_PATH = os.path.join(HERE, "libmindspeed_amd_trace.so")   # diagnostic variant: per-tile time stamps
 
 ARCH = "gfx950"
 # packed-fp32 VALU forms are switched off for every device translation unit.
@@ -52,13 +53,13 @@ def source_hash() -> str:
     return h.hexdigest()[:16]
 
 
-def _compile(src: str, force: bool) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
+def _compile(src: str, force: bool, extra=(), suffix="") -> str:
+    obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + suffix + ".o")
     deps = [src, os.path.join(HERE, "..", "include", "mindspeed_amd.h")]
     deps += [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) > os.path.getmtime(d) for d in deps):
         return obj
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", src, "-o", obj]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", src, "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{res.stderr}")
@@ -80,5 +81,24 @@ def build(force: bool = True, verbose: bool = False) -> str:
     return LIB_PATH
 
 
+def build_trace(verbose: bool = False) -> str:
+    """The diagnostic variant of the library: the grouped-matmul fast kernels compiled with MS_TRACE_TILES (every
+    workgroup records time stamps of its phases, read back with ms_trace_read; see profile_tools timeline).  Not
+    loaded by anything else; select it with MINDSPEED_AMD_LIB."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    objs = [_compile(s, True, ("-DMS_TRACE_TILES",), "_trace") if s.endswith("gmm_fast.hip") else _compile(s, False)
+            for s in sources()]
+    cmd = [_hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", TRACE_LIB_PATH, *objs]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stderr}")
+    if verbose:
+        print(f"built {TRACE_LIB_PATH}")
+    return TRACE_LIB_PATH
+
+
 if __name__ == "__main__":
-    build(force="--incremental" not in sys.argv, verbose=True)
+    if "--trace" in sys.argv:
+        build_trace(verbose=True)
+    else:
+        build(force="--incremental" not in sys.argv, verbose=True)

@@ -33,6 +33,20 @@
 
 #include "gmm_common.h"
 
+#ifdef MS_TRACE_TILES
+// Diagnostic build only (python -m mindspeed_amd.build --trace): every workgroup of the fast kernels records when it
+// started, found its tile, had its first operands in LDS, left the K loop and finished (100 MHz wall clock), plus the
+// compute unit it ran on; ms_trace_read copies the records of the last launches out.  The record of workgroup b is
+// slot b % kTraceSlots, so a launch with more workgroups than that overwrites its own early records.
+namespace ms {
+constexpr int kTraceSlots = 16384;
+__device__ long long g_tile_trace[kTraceSlots * 8];
+}  // namespace ms
+#define MS_TRACE(i) do { if (threadIdx.x == 0) ms::g_tile_trace[(blockIdx.x % ms::kTraceSlots) * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define MS_TRACE(i)
+#endif
+
 namespace ms {
 namespace {
 
@@ -353,6 +367,7 @@ __device__ __forceinline__ void ring_k_loop(const GmmArgs &p, const TileCoord &t
         request_done();
     }
     arrive();
+    MS_TRACE(3);
     read_frags(lds, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
 
@@ -494,6 +509,7 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
                 for (int part = 0; part < 4; ++part) load_part(std::true_type{}, part, red_len - BK);
             }
             lds_barrier();
+            MS_TRACE(3);
             read_frags(lds, 0, 0);
         }
 
@@ -552,6 +568,7 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
 
     // Epilogue.  acc[i][j][4*q+e] = C[row0 + wm*TM*32 + i*32 + (lane&31)]
     //                                [col0 + wn*TN*32 + j*32 + 8*q + 4*(lane>>5) + e]
+    MS_TRACE(4);
     const int64_t ldc = p.c_stride_row;
     constexpr int WR = TM * 32, WC = TN * 32;       // this wavefront's block of the tile
     if constexpr (OUT == OUT_SAME || OUT == OUT_SWIGLU || OUT == OUT_SWIGLU_GRAD) {
@@ -733,11 +750,23 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
 template <int DT, bool A_RED, bool B_RED, int OUT>
 __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
+    MS_TRACE(1);
     const TileCoord tc = locate_tile(p.table);
     if (!tc.valid) return;
+    MS_TRACE(2);
     if (tc.tile_rows == 256) gmm16_tile<DT, A_RED, B_RED, OUT, 256>(p, tc, lds);
     else if (tc.tile_rows == 128) gmm16_tile<DT, A_RED, B_RED, OUT, 128>(p, tc, lds);
     else gmm16_tile<DT, A_RED, B_RED, OUT, 64>(p, tc, lds);
+#ifdef MS_TRACE_TILES
+    if (threadIdx.x == 0) {
+        unsigned hw_id, xcc_id;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw_id));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_id));
+        long long *rec = g_tile_trace + (blockIdx.x % kTraceSlots) * 8;
+        rec[0] = (static_cast<long long>(xcc_id & 0xf) << 32) | ((hw_id >> 8) & 0xff) | (1ll << 40);   // XCC, CU/SH/SE bits, "valid"
+        rec[5] = wall_clock64();
+    }
+#endif
 }
 
 template <int DT, int OUT>
@@ -788,3 +817,18 @@ int launch_gmm16_fast(hipStream_t stream, const GmmArgs &args, int dtype, int ou
 }
 
 }  // namespace ms
+
+#ifdef MS_TRACE_TILES
+// Diagnostic builds only: ms_trace_clear zeroes the tile trace (call it before the launch to be looked at: records of
+// earlier, larger launches would otherwise remain), ms_trace_read copies its first n values (8 per record) to host memory.
+extern "C" int ms_trace_clear(void) {
+    static long long zeros[ms::kTraceSlots * 8];
+    if (hipDeviceSynchronize() != hipSuccess) return MS_ERR_HIP;
+    return hipMemcpyToSymbol(HIP_SYMBOL(ms::g_tile_trace), zeros, sizeof(zeros)) == hipSuccess ? MS_OK : MS_ERR_HIP;
+}
+
+extern "C" int ms_trace_read(long long *host, int n) {
+    if (n < 0 || n > ms::kTraceSlots * 8) return MS_ERR_INVALID_ARGUMENT;
+    return hipMemcpyFromSymbol(host, HIP_SYMBOL(ms::g_tile_trace), sizeof(long long) * n) == hipSuccess ? MS_OK : MS_ERR_HIP;
+}
+#endif

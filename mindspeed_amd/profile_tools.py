@@ -3,6 +3,7 @@
     python -m mindspeed_amd.profile_tools traffic --fetch F.csv --write W.csv [--workload mixtral] [--out FILE.json]
     python -m mindspeed_amd.profile_tools counters CSV [CSV ...]
     python -m mindspeed_amd.profile_tools power [--seconds 4] [--modes fwd1,dx1,dw1,library] [--data randn,zeros]
+    MINDSPEED_AMD_LIB=mindspeed_amd/libmindspeed_amd_trace.so python -m mindspeed_amd.profile_tools timeline [--modes ...] [--data ...]
 
 ``traffic`` reads the ``*_counter_collection.csv`` files of two ``rocprofv3 --pmc`` runs of ``bench.py`` (one with
 FETCH_SIZE, one with WRITE_SIZE; both with ``--copy-calibration MIB`` so that the plain copy kernel of known size is
@@ -15,6 +16,11 @@ sources they belong to (``bench.py`` reports them as ``roofline.traffic`` as lon
 ``power`` runs one grouped-matmul launch of the Mixtral-shape expert MLP back to back for a few seconds per
 (product, operand values) pair while a thread samples the board's power draw and shader clock from the amdgpu
 hwmon / sysfs files (read-only), and prints rate, power and clock side by side.
+
+``timeline`` needs the diagnostic build of the library (``python -m mindspeed_amd.build --trace``, selected with
+MINDSPEED_AMD_LIB): it launches one grouped matmul of the same shapes, reads the per-workgroup time stamps back and
+prints how a tile's time splits into finding the tile, waiting for the first operands, the K loop and the epilogue,
+and how long a compute unit stands idle between two workgroups.
 """
 from __future__ import annotations
 
@@ -236,6 +242,97 @@ def cmd_power(args):
             time.sleep(1.0)
 
 
+def _products(dev, data, gen):
+    """fc1-shaped products of the Mixtral expert MLP: name -> (callable, flops)."""
+    import torch
+
+    from .ops.gmm import gmm_raw
+
+    T, H, F, E = 8192, 4096, 14336, 8
+    bf = torch.bfloat16
+    counts = torch.full((E,), T // E, dtype=torch.int64, device=dev)
+
+    def operand(*shape):
+        if data == "zeros":
+            return torch.zeros(*shape, device=dev, dtype=bf)
+        return torch.randn(*shape, generator=gen, device=dev).to(bf)
+
+    def make(mode):
+        if mode == "fwd1":
+            x, w = operand(T, H), operand(E, H, 2 * F)
+            return lambda: gmm_raw(x, w, counts, 0, 1)
+        if mode == "dx1":
+            dy, w = operand(T, 2 * F), operand(E, H, 2 * F)
+            return lambda: gmm_raw(dy, w.transpose(1, 2), counts, 0, 1)
+        if mode == "dw1":
+            x, dy = operand(T, H), operand(T, 2 * F)
+            return lambda: gmm_raw(x.t(), dy, counts, 2, 1)
+        raise SystemExit(f"unknown mode {mode}")
+    return make, 2 * T * H * 2 * F
+
+
+def cmd_timeline(args):
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    from . import _lib
+
+    if not torch.cuda.is_available():
+        raise SystemExit("needs a HIP device")
+    lib = _lib.load()
+    if not hasattr(lib, "ms_trace_read"):
+        raise SystemExit("this library has no tile trace: build it with `python -m mindspeed_amd.build --trace` and "
+                         "select it with MINDSPEED_AMD_LIB=mindspeed_amd/libmindspeed_amd_trace.so")
+    lib.ms_trace_read.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    lib.ms_trace_read.restype = ctypes.c_int
+    lib.ms_trace_clear.argtypes = []
+    lib.ms_trace_clear.restype = ctypes.c_int
+    dev = torch.device("cuda", 0)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    slots = 16384
+    print("Mixtral-shape fc1 products (8192 rows in 8 equal groups, hidden 4096, 2*ffn 28672, bf16), one launch each; "
+          "times in microseconds from a 100 MHz clock, averaged over the workgroups that held a tile")
+    print(f"{'product':8s} {'operands':8s} {'tiles':>6s} {'find tile':>10s} {'first data':>11s} {'K loop':>9s} {'epilogue':>9s} "
+          f"{'tile total':>11s} {'idle gap':>9s} {'launch span':>12s} {'MFMA share':>11s}")
+    for data in args.data.split(","):
+        make, flops = _products(dev, data, gen)
+        for mode in args.modes.split(","):
+            fn = make(mode)
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            _lib.check(lib.ms_trace_clear(), "ms_trace_clear")
+            fn()
+            torch.cuda.synchronize()
+            buf = (ctypes.c_longlong * (slots * 8))()
+            _lib.check(lib.ms_trace_read(buf, slots * 8), "ms_trace_read")
+            rec = np.frombuffer(buf, dtype=np.int64).reshape(-1, 8)
+            rec = rec[(rec[:, 0] >> 40) == 1]
+            rec = rec[rec[:, 4] > rec[:, 1]]          # workgroups that held a tile
+            if len(rec) == 0:
+                print(f"{mode:8s} {data:8s} no records")
+                continue
+            us = lambda a, b: float((rec[:, a] - rec[:, b]).mean()) / 100.0     # noqa: E731
+            gaps = []
+            by_cu = {}
+            for r in rec:
+                by_cu.setdefault(int(r[0]) & ((1 << 40) - 1), []).append((int(r[1]), int(r[5])))
+            for runs in by_cu.values():
+                runs.sort()
+                gaps += [b[0] - a[1] for a, b in zip(runs, runs[1:])]
+            span = float(rec[:, 5].max() - rec[:, 1].min()) / 100.0
+            # MFMA time of a 256 x 256 tile: 2 * 256 * 256 * K flops at 1024 flop / clock / SIMD x 4 SIMDs, 2.4 GHz
+            tiles_total = len(rec)
+            mfma_us = flops / tiles_total / (4 * 1024 * 2.4e9) * 1e6
+            total = us(5, 1)
+            print(f"{mode:8s} {data:8s} {tiles_total:6d} {us(2, 1):10.2f} {us(3, 2):11.2f} {us(4, 3):9.2f} {us(5, 4):9.2f} "
+                  f"{total:11.2f} {(sum(gaps) / len(gaps) / 100.0) if gaps else float('nan'):9.2f} {span:12.1f} "
+                  f"{mfma_us / total:11.3f}", flush=True)
+            del fn
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
@@ -251,8 +348,11 @@ def main():
     w.add_argument("--seconds", type=float, default=4.0)
     w.add_argument("--modes", default="fwd1,dx1,dw1,library")
     w.add_argument("--data", default="randn,small,zeros")
+    tl = sub.add_parser("timeline")
+    tl.add_argument("--modes", default="fwd1,dx1,dw1")
+    tl.add_argument("--data", default="randn,zeros")
     args = ap.parse_args()
-    {"traffic": cmd_traffic, "counters": cmd_counters, "power": cmd_power}[args.cmd](args)
+    {"traffic": cmd_traffic, "counters": cmd_counters, "power": cmd_power, "timeline": cmd_timeline}[args.cmd](args)
 
 
 if __name__ == "__main__":

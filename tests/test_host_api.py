@@ -220,3 +220,13 @@ def test_shapes_propagate_on_meta_tensors():
     assert back.shape == (T, H)
     back.sum().backward()
     assert mprobs.grad.shape == (T, E)
+
+
+def test_probe_sources_and_trace_build_are_wired():
+    """The hardware probes are listed by their runner, and the diagnostic (tile trace) build has its own output path."""
+    from mindspeed_amd import build
+    from mindspeed_amd.probes import __main__ as probes
+
+    assert probes.names() == ["issue_cost", "lds_rates", "mfma_power"]
+    assert build.TRACE_LIB_PATH != build.LIB_PATH and build.TRACE_LIB_PATH.endswith("libmindspeed_amd_trace.so")
+    assert callable(build.build_trace)
