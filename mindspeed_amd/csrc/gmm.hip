@@ -140,6 +140,7 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
     table->slots_per_xcd = tiles;
     table->num_entries = n;
     for (int i = 0; i < 8; ++i) table->zeros[i] = 0;
+    for (int i = 0; i < 16; ++i) table->begins[i] = i < n ? table->entries[i].tile_begin : 0x7fffffff;
 }
 
 // 8 contiguous 16-bit elements starting at p; elements >= nvalid read as zero.
