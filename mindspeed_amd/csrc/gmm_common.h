@@ -96,16 +96,17 @@ __device__ __forceinline__ TileCoord locate_tile(const TileTable *table) {
     // for 32 tiles; with many row tiles (the weight gradient: hidden / 256 of them) plain row-tile-fastest order
     // would have them on 16 x 2 tiles and fetch 18.  Up to 4 row tiles per group the two orders are the same.
     {
+        constexpr int BR = 4, BC = 8;      // measured against 8 x 4, 8 x 8, 2 x 16 and 4 x 16: the fastest for all three products
         const int R = tc.e.num_row_tiles, C = tc.e.num_tiles / R;
-        const int cg = r / (8 * R);
-        const int rem = r - cg * 8 * R;
-        const int wc = C - 8 * cg < 8 ? C - 8 * cg : 8;        // column panels in this set
-        const int rb = rem / (4 * wc);
-        const int rem2 = rem - rb * 4 * wc;
-        const int hr = R - 4 * rb < 4 ? R - 4 * rb : 4;        // row tiles in this block
+        const int cg = r / (BC * R);
+        const int rem = r - cg * BC * R;
+        const int wc = C - BC * cg < BC ? C - BC * cg : BC;    // column panels in this set
+        const int rb = rem / (BR * wc);
+        const int rem2 = rem - rb * BR * wc;
+        const int hr = R - BR * rb < BR ? R - BR * rb : BR;    // row tiles in this block
         const int lc = rem2 / hr;
-        tc.col_tile = 8 * cg + lc;
-        tc.row_tile = 4 * rb + (rem2 - lc * hr);
+        tc.col_tile = BC * cg + lc;
+        tc.row_tile = BR * rb + (rem2 - lc * hr);
     }
     tc.tile_rows = (tc.e.tail_rows != 0 && tc.row_tile == tc.e.num_row_tiles - 1) ? tc.e.tail_rows : tc.e.tile_rows;
     tc.valid = true;
