@@ -91,6 +91,10 @@ GMM_CASES = [
     (37, 19, 23, 5, "random"),            # tiny and odd: element-wise paths
     (96, 20, 16, 3, "random"),            # dX writes 20 columns: a multiple of 4 but not of 8
     (256, 72, 44, 2, "equal"),            # forward writes 44 columns (n % 8 == 4) from vector-aligned operands
+    # tile order in 4 x 8 blocks with partly filled blocks on both sides: 6 / 7 row tiles and 9 column panels in
+    # forward, 6 x 9 in the weight gradient; 11 row tiles x 17 column panels (4 + 4 + 3, 8 + 8 + 1) in the last one
+    (3000, 1536, 2304, 2, "random"),
+    (2600, 1280, 4352, 1, "equal"),
 ]
 
 
