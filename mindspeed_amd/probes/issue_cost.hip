@@ -10,6 +10,7 @@
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef unsigned u4 __attribute__((ext_vector_type(4)));
 typedef int i4 __attribute__((ext_vector_type(4)));
+typedef unsigned u2 __attribute__((ext_vector_type(2)));
 
 template <int KIND, int NL, int MF, int WAVES>   // MF: 0 = 16x16x32, 1 = 32x32x16; WAVES: 4 (one per SIMD) or 8 (two per SIMD, half the MFMAs each)
 __global__ __launch_bounds__(WAVES * 64) void mix(long long *out, const u4 *g, int iters) {
@@ -60,10 +61,16 @@ __global__ __launch_bounds__(WAVES * 64) void mix(long long *out, const u4 *g, i
                 if constexpr (KIND == 7) asm volatile("ds_write_b128 %0, %1" :: "v"(voff + i * 1024), "v"(fa) : "memory");
                 if constexpr (KIND == 8) asm volatile("ds_write_b64 %0, %1" :: "v"(voff + i * 1024), "v"(*reinterpret_cast<__attribute__((ext_vector_type(2))) unsigned *>(&fa)) : "memory");
                 if constexpr (KIND == 9) asm volatile("v_add_u32 %0, %0, %1\n" : "+v"(sink) : "v"(voff));
+                if constexpr (KIND == 13) asm volatile("ds_read_b128 %0, %1" : "=v"(rg[i]) : "v"(voff + (i % 16) * 1024));
+                if constexpr (KIND == 14) {
+                    u2 t;
+                    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(t) : "v"(voff / 2 + (i % 16) * 512));
+                    rg[i][0] = t[0]; rg[i][1] = t[1];
+                }
             }
         }
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        if constexpr (KIND == 1 || KIND == 2 || KIND == 5 || KIND == 11 || KIND == 12) { for (int i = 0; i < NL; ++i) sink ^= rg[i][0]; }
+        if constexpr (KIND == 1 || KIND == 2 || KIND == 5 || KIND == 11 || KIND == 12 || KIND == 13 || KIND == 14) { for (int i = 0; i < NL; ++i) sink ^= rg[i][0]; }
     }
     long long t1 = clock64();
     float s = 0;
@@ -100,6 +107,10 @@ int main() {
     run<3, 16, 1>("32x32x16: m0 + global_load_lds_dwordx4 v64, off", o, g);
     run<7, 16, 1>("32x32x16: ds_write_b128", o, g);
     run<0, 0, 1>("32x32x16: MFMA only", o, g);
+    run<13, 16, 1>("32x32x16: ds_read_b128", o, g);
+    run<14, 32, 1>("32x32x16: ds_read_b64_tr_b16 x32", o, g);
+    run<13, 16, 0>("16x16x32: ds_read_b128", o, g);
+    run<14, 32, 0>("16x16x32: ds_read_b64_tr_b16 x32", o, g);
     run<11, 16, 1>("32x32x16: global_load_dwordx4, four bursts of four", o, g);
     run<12, 16, 1>("32x32x16: global_load_dwordx4, two bursts of eight", o, g);
     run<11, 16, 0>("16x16x32: global_load_dwordx4, four bursts of four", o, g);
