@@ -184,6 +184,16 @@ int ms_moe_routing_map_probs_grad(ms_stream_t stream, const int32_t *row_id_map,
  * accumulate != 0: y += result (requires out_dtype == MS_FP32).
  * ---------------------------------------------------------------------- */
 int ms_gmm_workspace_size(int64_t num_groups, int64_t m, int group_type, size_t *bytes);
+/* The second form of the workspace query (the GetWorkspaceSize half of the two-phase aclnnGroupedMatmul
+ * call, aclnn_common.h:587-644, sees all operands too): at least ms_gmm_workspace_size, and up to 32 MiB
+ * more where ms_gmm may then split the reduction of small tail tiles.  That applies to group_type 0 with a
+ * 16-bit output when the launch has few rounds of tiles and k >= 4096: the 64- / 128-row tile that ends a
+ * ragged group is computed in up to 4 parts along k (fp32 partial sums in the workspace, added in part
+ * order and rounded once by a second small kernel), so that the last round of the launch does not leave
+ * most compute units waiting for a few long tiles.  With the smaller workspace ms_gmm runs unsplit; results of
+ * the two differ by the rounding of the summation order in the rows of those tail tiles only. */
+int ms_gmm_workspace_size_split(int64_t num_groups, int64_t m, int64_t k, int64_t n, int group_type,
+                                int dtype, int out_dtype, int accumulate, size_t *bytes);
 int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1,
            const void *weight, int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1,
            void *y, int64_t y_stride_row, const int64_t *group_list, int group_list_type,
@@ -192,9 +202,10 @@ int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_strid
 
 /* ms_gmm for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): the same arguments without the workspace pair, the same
- * kernels and results.  It has no counterpart in the reference, whose shims always draw a workspace
+ * kernels and the results of ms_gmm with the workspace of ms_gmm_workspace_size (tail tiles are never
+ * split).  It has no counterpart in the reference, whose shims always draw a workspace
  * from the framework's allocator.  The tile table lives in a fixed device array inside the library
- * (about 120 KB per GPU, held until the process ends), which bounds num_groups to 1024; more groups
+ * (about 340 KB per GPU, held until the process ends), which bounds num_groups to 1024; more groups
  * report MS_ERR_UNSUPPORTED.  The call allocates and frees nothing.  The first call on a device looks
  * the array's address up (hipGetSymbolAddress), so make that call outside a graph capture.  All calls
  * on one GPU share the array: calls that may overlap on one GPU (different streams, different

@@ -7,7 +7,11 @@
 //     per-group tile ranges (no host read of group_list, empty groups emit no
 //     row tiles, a trailing pseudo-group zero-fills rows past the last offset;
 //     ragged groups may end in a 64- or 128-row tile; per-group weight offsets
-//     may come from a list of separately allocated matrices).
+//     may come from a list of separately allocated matrices).  In launches with
+//     few rounds of tiles those small tiles run last, and with room in the
+//     workspace their reduction is cut into parts (fp32 partial sums, added up
+//     by gmm_split_reduce_kernel) so that they fill one round instead of
+//     running long on a few compute units.
 //   * every XCD takes a contiguous eighth of every group's tiles (workgroup b
 //     runs on XCD b % 8), row-tile-fastest inside a column panel, so the
 //     workgroups running together on an XCD share operand panels in its L2.
@@ -18,6 +22,7 @@
 //     256x256x64 tile and 4x4 v_mfma_f32_32x32x16 per wavefront; and
 //     gmm32_kernel for fp32 inputs (v_mfma_f32_32x32x2f32, 128x128x8 tiles).
 #include <mutex>
+#include <type_traits>
 
 #include "gmm_common.h"
 
@@ -36,111 +41,276 @@ __global__ void gmm_weight_offsets_kernel(const WeightOffsets o, int n, int64_t 
 }
 
 // ---- schedule ------------------------------------------------------------------------
-// With split_tails the last row tile of a group may be a smaller one (64 or 128 rows, the smallest that
-// holds the remainder), so ragged groups do not pay for a whole extra tile.  part = 0: one entry for the
-// whole group; the small tile stays in the group's tile range, next to the full tiles of the same column
-// panel, so the weight panel it reads is being read by its neighbours at the same time.  part = 1 / 2: the
-// group's full tiles / its small tile as entries of their own (used when the small tiles of all groups are
-// scheduled after all full tiles).
-__device__ __forceinline__ int emit_rows(TileTable *table, int n, int &tiles, GroupEntry e, int tile_rows,
-                                         int num_col_tiles, int split_tails, int part) {
-    const int rows = e.row_end - e.row_begin;
-    if (rows <= 0) return n;
-    e.tile_rows = tile_rows;
-    e.num_row_tiles = (rows + tile_rows - 1) / tile_rows;
-    const int rem = rows - (e.num_row_tiles - 1) * tile_rows;      // rows of the last tile, 1..tile_rows
-    e.tail_rows = !split_tails ? 0 : (rem <= 64 ? 64 : (rem <= 128 ? 128 : 0));
-    if (part == 1 && e.tail_rows != 0) {
-        e.num_row_tiles -= 1;
-        e.row_end = e.row_begin + e.num_row_tiles * tile_rows;
-        e.tail_rows = 0;
-        if (e.num_row_tiles == 0) return n;
-    } else if (part == 2) {
-        if (e.tail_rows == 0) return n;
-        e.row_begin += (e.num_row_tiles - 1) * tile_rows;
-        e.num_row_tiles = 1;
-    }
-    e.num_tiles = e.num_row_tiles * num_col_tiles;
-    e.share = (e.num_tiles + 7) >> 3;
-    e.tile_begin = tiles;
-    tiles += e.share;
-    table->entries[n++] = e;
-    return n;
+// One workgroup turns the device-resident group list into the tile table.  Every thread takes a run of consecutive
+// groups; the running quantities (group end offsets, entry numbers, slot numbers, split-workspace blocks) come from
+// block-wide prefix scans, so the kernel's time does not grow with the number of groups the way a serial walk does.
+//
+// Entries.  With split_tails the last row tile of a group may be a smaller one (64 or 128 rows, the smallest that
+// holds the remainder), so ragged groups do not pay for a whole extra tile.  Normally a group is one entry and the
+// small tile stays in the group's tile range, next to the full tiles of the same column panel, so the weight panel
+// it reads is being read by its neighbours at the same time.  When the launch has only a few rounds of tiles (fewer
+// than tails_last_below tiles in all) the entries come in two passes: first every group's full tiles, then every
+// group's small tile as an entry of its own, so that the last, partly filled round is made of the short tiles.
+// With a split workspace (split_records != nullptr) the reduction of those last-scheduled small tiles is cut into up
+// to kMaxSplit ranges, as many as keep all parts of all tails within one round of the compute units: a small tile of
+// a long reduction otherwise runs as long as most of a full tile while a few compute units work and the others wait.
+// Each part is an entry that writes fp32 partial sums; gmm_split_reduce_kernel adds them up.
+// Split on the reduction dim: a tile's cost is its group's reduction length, so groups with an above-average length
+// come first (they start early on every XCD), the short ones fill in after.
+struct ScanItem {
+    int n0, slots0;      // entries and slots of the first pass
+    int n1, slots1;      // ... of the second pass
+    int tails, pairs;    // split tails and their (tail, part) blocks of the split workspace
+};
+__device__ __forceinline__ ScanItem operator+(const ScanItem &a, const ScanItem &b) {
+    return ScanItem{a.n0 + b.n0, a.slots0 + b.slots0, a.n1 + b.n1, a.slots1 + b.slots1, a.tails + b.tails, a.pairs + b.pairs};
 }
+
+// Exclusive prefix of v over the 256 threads of the workgroup (thread order) and the total; scratch holds 4 values.
+template <typename T, typename Op>
+__device__ __forceinline__ T block_scan_exclusive(T v, Op op, T identity, T *scratch, T &total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    T x = v;                                   // inclusive within the wavefront
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        T y;
+        static_assert(sizeof(T) % 4 == 0, "scan items are made of 32-bit words");
+        const int *src = reinterpret_cast<const int *>(&x);
+        int *dst = reinterpret_cast<int *>(&y);
+#pragma unroll
+        for (int w = 0; w < static_cast<int>(sizeof(T) / 4); ++w) dst[w] = __shfl_up(src[w], d, 64);
+        if (lane >= d) x = op(y, x);
+    }
+    __syncthreads();                           // scratch may still be read from an earlier scan
+    if (lane == 63) scratch[wave] = x;
+    __syncthreads();
+    T base = identity;
+    for (int w = 0; w < wave; ++w) base = op(base, scratch[w]);
+    total = op(op(scratch[0], scratch[1]), op(scratch[2], scratch[3]));
+    // exclusive: everything before this thread = base (+) the lanes before it in its wavefront
+    T before;
+    {
+        const int *src = reinterpret_cast<const int *>(&x);
+        int *dst = reinterpret_cast<int *>(&before);
+#pragma unroll
+        for (int w = 0; w < static_cast<int>(sizeof(T) / 4); ++w) dst[w] = __shfl_up(src[w], 1, 64);
+    }
+    return lane == 0 ? base : op(base, before);
+}
+
+// What one group contributes, and its entries.
+struct GroupPlan {
+    int row_tiles;       // row tiles of the group (split on rows) / of the output block (split on the reduction dim)
+    int tail_rows;       // 64 / 128 if the last row tile is a small one, else 0
+    int rem;             // rows of the last row tile
+    bool first_pass;     // split on the reduction dim: the group belongs to the first pass
+};
 
 __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__restrict__ group_list,
                                                            int group_list_type, int group_type, int num_groups,
                                                            int m, int k, int tile_rows, int num_col_tiles,
                                                            int split_tails, int tails_last_below,
                                                            int64_t b_stride_group, int64_t c_stride_group,
-                                                           const int64_t *__restrict__ b_offsets, TileTable *table) {
-    extern __shared__ int64_t gl[];
-    for (int g = threadIdx.x; g < num_groups; g += blockDim.x) gl[g] = group_list[g];
-    __syncthreads();
-    if (threadIdx.x != 0) return;
-    int tiles = 0;
-    int n = 0;
-    int64_t prev = 0;
-    // Split on the reduction dim: a tile's cost is its group's reduction length, so groups with an
-    // above-average length are emitted first (they start early on every XCD), the short ones fill in after.
-    //
-    // Split on rows with small tail tiles: when the launch has only a few rounds of tiles (fewer than
-    // tails_last_below tiles in all), the small tiles of all groups are scheduled after all full tiles, so
-    // that the last, partly filled round is made of the short tiles; with many rounds they stay next to
-    // their group's full tiles, where they find the group's weight panel in L2.
-    bool tails_last = false;
-    if (group_type == 0 && split_tails) {
-        int64_t total = 0, p0 = 0;
-        for (int g = 0; g < num_groups; ++g) {
-            int64_t end = group_list_type == 0 ? gl[g] : p0 + gl[g];
-            end = end < p0 ? p0 : end;
-            end = end > m ? m : end;
-            total += (end - p0 + tile_rows - 1) / tile_rows * num_col_tiles;
-            p0 = end;
-        }
-        tails_last = total < tails_last_below;
-    }
-    const int passes = (group_type == 2 || tails_last) ? 2 : 1;
-    const int64_t mean_len = num_groups > 0 ? m / num_groups : 0;
-    for (int pass = 0; pass < passes; ++pass) {
-        prev = 0;
-        for (int g = 0; g < num_groups; ++g) {
-            int64_t end = group_list_type == 0 ? gl[g] : prev + gl[g];
-            end = end < prev ? prev : end;
-            end = end > m ? m : end;
-            const bool is_long = end - prev >= mean_len;
-            if (passes == 1 || tails_last || is_long == (pass == 0)) {
-                GroupEntry e{};
-                if (group_type == 0) {
-                    e.row_begin = static_cast<int>(prev);
-                    e.row_end = static_cast<int>(end);
-                    e.red_begin = 0;
-                    e.red_end = k;
-                    e.b_off = b_offsets != nullptr ? b_offsets[g] : g * b_stride_group;
-                    e.c_off = 0;
-                } else {
-                    e.row_begin = 0;
-                    e.row_end = k;
-                    e.red_begin = static_cast<int>(prev);
-                    e.red_end = static_cast<int>(end);
-                    e.b_off = 0;
-                    e.c_off = g * c_stride_group;
-                }
-                n = emit_rows(table, n, tiles, e, tile_rows, num_col_tiles, split_tails, tails_last ? pass + 1 : 0);
+                                                           const int64_t *__restrict__ b_offsets, TileTable *table,
+                                                           SplitTail *split_records, int split_cols, int split_cus) {
+    extern __shared__ int64_t ends[];          // [num_groups] clamped end offset of every group
+    __shared__ int64_t scratch64[4];
+    __shared__ ScanItem scratch_item[4];
+    const int tid = threadIdx.x;
+    const int per = (num_groups + 255) >> 8;
+    const int g0 = tid * per < num_groups ? tid * per : num_groups;
+    const int g1 = g0 + per < num_groups ? g0 + per : num_groups;
+
+    // Group ends.  Cumulative list: end_g = min(m, max(0, list[0..g])); counts: end_g = min(m, sum of the counts so far,
+    // negative counts read as 0).  Both are what a walk with "never before the previous end, never past m" gives.
+    {
+        int64_t run = 0;
+        for (int g = g0; g < g1; ++g) {
+            int64_t v = group_list[g];
+            if (group_list_type == 0) {
+                run = v > run ? v : run;
+            } else {
+                v = v < 0 ? 0 : (v > m ? m : v);
+                run += v;
             }
-            prev = end;
+            ends[g] = run;
+        }
+        int64_t total;
+        const int64_t before = group_list_type == 0
+            ? block_scan_exclusive(run, [](int64_t a, int64_t b) { return a > b ? a : b; }, int64_t{0}, scratch64, total)
+            : block_scan_exclusive(run, [](int64_t a, int64_t b) { return a + b; }, int64_t{0}, scratch64, total);
+        for (int g = g0; g < g1; ++g) {
+            int64_t e = group_list_type == 0 ? (ends[g] > before ? ends[g] : before) : ends[g] + before;
+            ends[g] = e > m ? m : e;
         }
     }
-    if (group_type == 0 && prev < m) {  // rows past the last offset: zero-fill
-        GroupEntry e{};
-        e.row_begin = static_cast<int>(prev);
-        e.row_end = m;
-        n = emit_rows(table, n, tiles, e, tile_rows, num_col_tiles, split_tails, 0);
+    __syncthreads();
+
+    auto plan_of = [&](int g) {
+        const int prev = g > 0 ? static_cast<int>(ends[g - 1]) : 0;
+        const int len = static_cast<int>(ends[g]) - prev;              // rows (group_type 0) / reduction length
+        GroupPlan p{};
+        if (group_type == 0) {
+            p.row_tiles = (len + tile_rows - 1) / tile_rows;
+            p.rem = len - (p.row_tiles - 1) * tile_rows;
+            p.tail_rows = (!split_tails || len <= 0) ? 0 : (p.rem <= 64 ? 64 : (p.rem <= 128 ? 128 : 0));
+        } else {
+            p.row_tiles = (k + tile_rows - 1) / tile_rows;
+            p.rem = k - (p.row_tiles - 1) * tile_rows;
+            p.tail_rows = (!split_tails || k <= 0) ? 0 : (p.rem <= 64 ? 64 : (p.rem <= 128 ? 128 : 0));
+            p.first_pass = len >= (num_groups > 0 ? m / num_groups : 0);
+        }
+        return p;
+    };
+    auto share_of = [&](int row_tiles) { return (row_tiles * num_col_tiles + 7) >> 3; };
+
+    // Launch-wide decisions (split on rows only): do the small tiles go last, and in how many parts.
+    bool tails_last = false;
+    int split_parts = 1;
+    if (group_type == 0 && split_tails) {
+        ScanItem mine{};                       // n0: tiles, n1: groups with a small tail
+        for (int g = g0; g < g1; ++g) {
+            const GroupPlan p = plan_of(g);
+            mine.n0 += p.row_tiles * num_col_tiles;
+            mine.n1 += p.tail_rows != 0 ? 1 : 0;
+        }
+        ScanItem all;
+        block_scan_exclusive(mine, [](const ScanItem &a, const ScanItem &b) { return a + b; }, ScanItem{}, scratch_item, all);
+        const int total = all.n0, tails = all.n1;
+        tails_last = total < tails_last_below;
+        // Worth splitting only where the small tiles would otherwise end the launch by themselves: the full tiles'
+        // last round is complete, or leaves too few compute units free to run the small tiles (about half a full
+        // tile's time each) beside it.
+        const int tail_tiles = tails * num_col_tiles;
+        const int full = total - tail_tiles;
+        const int last = full % split_cus;
+        const int free_cus = last == 0 ? 0 : split_cus - last;
+        if (tails_last && split_records != nullptr && tails > 0 && full > 0 && tail_tiles > 2 * free_cus) {
+            split_parts = kSplitCus / tail_tiles;
+            if (split_parts > k / kSplitMinRed) split_parts = k / kSplitMinRed;
+            if (split_parts > kMaxSplit) split_parts = kMaxSplit;
+            if (split_parts < 2) split_parts = 1;
+        }
     }
-    table->slots_per_xcd = tiles;
-    table->num_entries = n;
-    for (int i = 0; i < 8; ++i) table->zeros[i] = 0;
-    for (int i = 0; i < 16; ++i) table->begins[i] = i < n ? table->entries[i].tile_begin : 0x7fffffff;
+    // parts of a split tail: equal ranges of whole K steps, none empty
+    const int steps = (k + BK - 1) / BK;
+    const int part_len = split_parts > 1 ? (steps + split_parts - 1) / split_parts * BK : k;
+    const int used_parts = split_parts > 1 ? (k + part_len - 1) / part_len : 1;
+
+    // What every group emits in each pass.
+    auto item_of = [&](const GroupPlan &p) {
+        ScanItem it{};
+        if (group_type == 2) {
+            if (p.row_tiles > 0) {
+                if (p.first_pass) { it.n0 = 1; it.slots0 = share_of(p.row_tiles); }
+                else { it.n1 = 1; it.slots1 = share_of(p.row_tiles); }
+            }
+        } else if (p.row_tiles > 0) {
+            if (!tails_last) {
+                it.n0 = 1; it.slots0 = share_of(p.row_tiles);
+            } else {
+                const int full_tiles = p.tail_rows != 0 ? p.row_tiles - 1 : p.row_tiles;
+                if (full_tiles > 0) { it.n0 = 1; it.slots0 = share_of(full_tiles); }
+                if (p.tail_rows != 0) {
+                    const int parts = split_parts > 1 ? used_parts : 1;
+                    it.n1 = parts; it.slots1 = parts * share_of(1);
+                    if (split_parts > 1) { it.tails = 1; it.pairs = parts; }
+                }
+            }
+        }
+        return it;
+    };
+    ScanItem mine{};
+    for (int g = g0; g < g1; ++g) mine = mine + item_of(plan_of(g));
+    ScanItem all;
+    ScanItem at = block_scan_exclusive(mine, [](const ScanItem &a, const ScanItem &b) { return a + b; }, ScanItem{}, scratch_item, all);
+
+    const int max_entries = (1 + kMaxSplit) * num_groups + 2;
+    auto put = [&](int idx, const GroupEntry &e) {
+        if (idx < max_entries) table->entries[idx] = e;
+        if (idx < 16) table->begins[idx] = e.tile_begin;
+    };
+    for (int g = g0; g < g1; ++g) {
+        const GroupPlan p = plan_of(g);
+        const ScanItem it = item_of(p);
+        const int prev = g > 0 ? static_cast<int>(ends[g - 1]) : 0;
+        const int end = static_cast<int>(ends[g]);
+        GroupEntry e{};
+        e.tile_rows = tile_rows;
+        if (group_type == 0) {
+            e.row_begin = prev; e.row_end = end; e.red_begin = 0; e.red_end = k;
+            e.b_off = b_offsets != nullptr ? b_offsets[g] : g * b_stride_group;
+            e.c_off = 0;
+        } else {
+            e.row_begin = 0; e.row_end = k; e.red_begin = prev; e.red_end = end;
+            e.b_off = 0;
+            e.c_off = g * c_stride_group;
+        }
+        if (it.n0 != 0) {                       // first pass: the whole group, or its full tiles
+            GroupEntry f = e;
+            const bool full_only = group_type == 0 && tails_last && p.tail_rows != 0;
+            f.num_row_tiles = full_only ? p.row_tiles - 1 : p.row_tiles;
+            f.tail_rows = full_only ? 0 : p.tail_rows;
+            if (full_only) f.row_end = f.row_begin + f.num_row_tiles * tile_rows;
+            f.num_tiles = f.num_row_tiles * num_col_tiles;
+            f.share = (f.num_tiles + 7) >> 3;
+            f.tile_begin = at.slots0;
+            put(at.n0, f);
+        }
+        if (it.n1 != 0) {                       // second pass
+            GroupEntry f = e;
+            if (group_type == 0) {              // the small tile, whole or in parts
+                f.row_begin = prev + (p.row_tiles - 1) * tile_rows;
+                f.num_row_tiles = 1;
+                f.tail_rows = p.tail_rows;
+            } else {
+                f.num_row_tiles = p.row_tiles;
+                f.tail_rows = p.tail_rows;
+            }
+            f.num_tiles = f.num_row_tiles * num_col_tiles;
+            f.share = (f.num_tiles + 7) >> 3;
+            if (it.tails != 0) {
+                if (at.tails < num_groups) split_records[at.tails] = SplitTail{f.row_begin, p.rem, at.pairs, it.n1};
+                for (int s = 0; s < it.n1; ++s) {
+                    f.red_begin = s * part_len;
+                    f.red_end = f.red_begin + part_len < k ? f.red_begin + part_len : k;
+                    f.split = s + 1;
+                    f.c_off = (static_cast<int64_t>(at.pairs + s) * kSplitRows - f.row_begin) * split_cols;
+                    f.tile_begin = all.slots0 + at.slots1 + s * f.share;
+                    put(all.n0 + at.n1 + s, f);
+                }
+            } else {
+                f.tile_begin = all.slots0 + at.slots1;
+                put(all.n0 + at.n1, f);
+            }
+        }
+        at = at + it;
+    }
+    if (tid == 0) {
+        int n = all.n0 + all.n1;
+        int slots = all.slots0 + all.slots1;
+        const int last_end = num_groups > 0 ? static_cast<int>(ends[num_groups - 1]) : 0;
+        if (group_type == 0 && last_end < m) {  // rows past the last offset: zero-fill (empty reduction range)
+            GroupEntry e{};
+            e.row_begin = last_end;
+            e.row_end = m;
+            e.tile_rows = tile_rows;
+            const int len = m - last_end;
+            e.num_row_tiles = (len + tile_rows - 1) / tile_rows;
+            const int rem = len - (e.num_row_tiles - 1) * tile_rows;
+            e.tail_rows = !split_tails ? 0 : (rem <= 64 ? 64 : (rem <= 128 ? 128 : 0));
+            e.num_tiles = e.num_row_tiles * num_col_tiles;
+            e.share = (e.num_tiles + 7) >> 3;
+            e.tile_begin = slots;
+            slots += e.share;
+            put(n++, e);
+        }
+        table->slots_per_xcd = slots;
+        table->num_entries = n;
+        table->num_split_tails = all.tails;
+        for (int i = 0; i < 8; ++i) table->zeros[i] = 0;
+        for (int i = n; i < 16; ++i) table->begins[i] = 0x7fffffff;
+    }
 }
 
 // 8 contiguous 16-bit elements starting at p; elements >= nvalid read as zero.
@@ -454,11 +624,73 @@ int current_device_cus() {
 }
 
 constexpr size_t table_bytes(int64_t num_groups) {
-    return sizeof(TileTable) + static_cast<size_t>(2 * num_groups + 2) * sizeof(GroupEntry);   // full + tail entries
+    // per group: its full tiles, its tail tile in up to kMaxSplit parts; plus the zero-fill pseudo-group
+    return sizeof(TileTable) + static_cast<size_t>((1 + kMaxSplit) * num_groups + 2) * sizeof(GroupEntry);
 }
-// workspace = tile table, then (8-byte aligned) room for the per-group weight offsets of the list form
+// workspace = tile table, then (8-byte aligned) room for the per-group weight offsets of the list form, then the
+// records of the split tails
 constexpr size_t offsets_pos(int64_t num_groups) { return (table_bytes(num_groups) + 7) & ~static_cast<size_t>(7); }
-constexpr size_t workspace_need(int64_t num_groups) { return offsets_pos(num_groups) + kMaxWeightList * sizeof(int64_t); }
+constexpr size_t split_records_pos(int64_t num_groups) { return offsets_pos(num_groups) + kMaxWeightList * sizeof(int64_t); }
+constexpr size_t workspace_need(int64_t num_groups) {
+    return split_records_pos(num_groups) + static_cast<size_t>(num_groups) * sizeof(SplitTail);
+}
+// ... and, for launches that may split the reduction of their small tail tiles, the fp32 partial sums behind that
+constexpr size_t split_ws_pos(int64_t num_groups) { return (workspace_need(num_groups) + 255) & ~static_cast<size_t>(255); }
+
+// Whether a launch of these sizes can come to split its tail tiles at all (the schedule kernel decides from the
+// group list whether it does), and how many bytes of partial sums it may then write: the parts of a launch number at
+// most kSplitCus tiles, i.e. kSplitCus / column tiles blocks of kSplitRows x n floats.
+bool may_split_tails(int64_t m, int64_t k, int64_t n, int group_type, int dtype, int out_dtype, int accumulate,
+                     int num_cus) {
+    if (group_type != 0 || dtype == MS_FP32 || out_dtype != dtype || accumulate) return false;
+    const int64_t col_tiles = ceil_div(n, BN);
+    // (the schedule kernel splits only when at least three quarters of a round of full tiles run in front)
+    return k >= 2 * kSplitMinRed && 2 * col_tiles <= kSplitCus && n % 8 == 0 &&
+           ceil_div(m, BM) * col_tiles < static_cast<int64_t>(kTailsLastRounds) * num_cus &&
+           4 * ceil_div(m, 128) * col_tiles >= 3 * static_cast<int64_t>(num_cus);
+}
+size_t split_ws_bytes(int64_t n) {
+    const int64_t pairs = kSplitCus / ceil_div(n, BN);
+    return static_cast<size_t>(pairs) * kSplitRows * static_cast<size_t>(n) * sizeof(float);
+}
+
+// y[row, :] of every split tail = the sum of its parts' partial sums (in part order), rounded once.
+// grid (num_groups, ceil(n / 2048), 16): block (j, c, z) takes rows z, z + 16, ... of tail j, 8 columns per lane.
+template <int DT>
+__global__ __launch_bounds__(256) void gmm_split_reduce_kernel(const TileTable *__restrict__ table,
+                                                               const SplitTail *__restrict__ tails,
+                                                               const float *__restrict__ ws, uint16_t *__restrict__ y,
+                                                               int64_t ldy, int n) {
+    if (static_cast<int>(blockIdx.x) >= table->num_split_tails) return;
+    const SplitTail t = tails[blockIdx.x];
+    const int col = (blockIdx.y * 256 + threadIdx.x) * 8;
+    if (col >= n) return;
+    using DTT = std::conditional_t<DT == MS_BF16, BF16, FP16>;
+    for (int r = blockIdx.z; r < t.rows; r += gridDim.z) {
+        // all parts requested at once (a part past the last one re-reads part 0 and is left out of the sum)
+        f32x4 pl[kMaxSplit], ph[kMaxSplit];
+#pragma unroll
+        for (int s = 0; s < kMaxSplit; ++s) {
+            const float *src = ws + (static_cast<int64_t>(t.pair0 + (s < t.parts ? s : 0)) * kSplitRows + r) * n + col;
+            pl[s] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src));
+            ph[s] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src + 4));
+        }
+        f32x4 lo = pl[0], hi = ph[0];
+#pragma unroll
+        for (int s = 1; s < kMaxSplit; ++s)
+            if (s < t.parts) {
+                lo += pl[s];
+                hi += ph[s];
+            }
+        uint16_t o[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            o[e] = DTT::from_float(lo[e]);
+            o[4 + e] = DTT::from_float(hi[e]);
+        }
+        *reinterpret_cast<v16 *>(y + static_cast<int64_t>(t.row_begin + r) * ldy + col) = *reinterpret_cast<v16 *>(o);
+    }
+}
 
 template <int DT, int OUT>
 int launch16(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red, unsigned grid) {
@@ -488,6 +720,16 @@ extern "C" int ms_gmm_workspace_size(int64_t num_groups, int64_t m, int group_ty
     MS_REQUIRE(num_groups >= 1 && num_groups <= kMaxGroups, MS_ERR_UNSUPPORTED,
                "ms_gmm_workspace_size: num_groups %lld outside [1, %d]", (long long)num_groups, kMaxGroups);
     *bytes = (workspace_need(num_groups) + 255) & ~static_cast<size_t>(255);
+    return MS_OK;
+}
+
+extern "C" int ms_gmm_workspace_size_split(int64_t num_groups, int64_t m, int64_t k, int64_t n, int group_type, int dtype,
+                                           int out_dtype, int accumulate, size_t *bytes) {
+    if (int rc = ms_gmm_workspace_size(num_groups, m, group_type, bytes)) return rc;
+    MS_REQUIRE(m >= 0 && k >= 0 && n >= 0, MS_ERR_INVALID_ARGUMENT, "ms_gmm_workspace_size_split: bad sizes m=%lld k=%lld n=%lld",
+               (long long)m, (long long)k, (long long)n);
+    if (may_split_tails(m, k, n, group_type, dtype, out_dtype, accumulate, kSplitCus))
+        *bytes = (split_ws_pos(num_groups) + split_ws_bytes(n) + 255) & ~static_cast<size_t>(255);
     return MS_OK;
 }
 
@@ -586,11 +828,23 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
                            static_cast<int>(num_groups), b_offsets);
         MS_CHECK_LAUNCH("gmm_weight_offsets_kernel");
     }
+    // Splitting the reduction of small tail tiles needs the larger workspace of ms_gmm_workspace_size_split; with the
+    // plain one the launch runs unsplit.
+    SplitTail *split_records = nullptr;
+    float *split_ws = nullptr;
+    if (swiglu == nullptr && swiglu_grad == nullptr &&
+        may_split_tails(m, k, n, group_type, dtype, out_dtype, accumulate, num_cus) &&
+        workspace_bytes >= split_ws_pos(num_groups) + split_ws_bytes(n) &&
+        (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
+        split_records = reinterpret_cast<SplitTail *>(static_cast<char *>(workspace) + split_records_pos(num_groups));
+        split_ws = reinterpret_cast<float *>(static_cast<char *>(workspace) + split_ws_pos(num_groups));
+    }
     auto schedule = [&](int split_tails) -> int {
         hipLaunchKernelGGL(gmm_schedule_kernel, dim3(1), dim3(256), static_cast<size_t>(num_groups) * sizeof(int64_t),
                            stream, group_list, group_list_type, group_type, static_cast<int>(num_groups),
                            static_cast<int>(m), static_cast<int>(k), tile_rows, static_cast<int>(num_col_tiles),
-                           split_tails, kTailsLastRounds * num_cus, w_stride_group, c_stride_group, b_offsets, table);
+                           split_tails, kTailsLastRounds * num_cus, w_stride_group, c_stride_group, b_offsets, table,
+                           split_tails ? split_records : nullptr, static_cast<int>(n), num_cus);
         MS_CHECK_LAUNCH("gmm_schedule_kernel");
         return MS_OK;
     };
@@ -607,7 +861,11 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     args.c_stride_row = y_stride_row;
     args.cols = static_cast<int>(n);
     args.num_col_tiles = static_cast<int>(num_col_tiles);
-    const unsigned grid = static_cast<unsigned>((ceil_div(tiles_bound, 8) + 2 * num_groups + 2) * 8);
+    // slots per XCD: every entry rounds its tiles up to a multiple of 8; a launch that may split its tail tiles has up
+    // to kMaxSplit entries per tail and up to kSplitCus more tiles
+    const unsigned grid = split_ws == nullptr
+        ? static_cast<unsigned>((ceil_div(tiles_bound, 8) + 2 * num_groups + 2) * 8)
+        : static_cast<unsigned>((ceil_div(tiles_bound + kSplitCus, 8) + (1 + kMaxSplit) * num_groups + 2) * 8);
 
     if (swiglu != nullptr) {
         args.cols = static_cast<int>(n / 2);
@@ -692,7 +950,21 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
         return launch_gmm16_fast(stream, args, dtype, OUT_SWIGLU_GRAD, true, true, grid);
     }
     if (int rc = schedule(fast ? 1 : 0)) return rc;
-    if (fast) return launch_gmm16_fast(stream, args, dtype, out, a_is_red, b_is_red, grid);
+    if (fast) {
+        args.split_ws = split_ws;
+        if (int rc = launch_gmm16_fast(stream, args, dtype, out, a_is_red, b_is_red, grid)) return rc;
+        if (split_ws != nullptr) {
+            const dim3 rgrid(static_cast<unsigned>(num_groups), static_cast<unsigned>(ceil_div(n, 2048)), 16);
+            if (dtype == MS_BF16)
+                hipLaunchKernelGGL(gmm_split_reduce_kernel<MS_BF16>, rgrid, dim3(256), 0, stream, table, split_records,
+                                   split_ws, static_cast<uint16_t *>(y), y_stride_row, static_cast<int>(n));
+            else
+                hipLaunchKernelGGL(gmm_split_reduce_kernel<MS_FP16>, rgrid, dim3(256), 0, stream, table, split_records,
+                                   split_ws, static_cast<uint16_t *>(y), y_stride_row, static_cast<int>(n));
+            MS_CHECK_LAUNCH("gmm_split_reduce_kernel");
+        }
+        return MS_OK;
+    }
     if (dtype == MS_BF16) {
         if (out == OUT_SAME) return launch16<MS_BF16, OUT_SAME>(stream, args, a_is_red, b_is_red, grid);
         if (out == OUT_F32) return launch16<MS_BF16, OUT_F32>(stream, args, a_is_red, b_is_red, grid);

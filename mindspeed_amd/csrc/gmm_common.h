@@ -21,14 +21,29 @@ struct GroupEntry {
     int tail_rows;           // rows of the group's last row tile if it is a smaller one (64 / 128), else 0
     int num_tiles;           // num_row_tiles * column tiles
     int share;               // ceil(num_tiles / 8): tiles of this group handled by each XCD
+    int split;               // 0, or 1 + the part number of a small tail tile whose reduction is split: such a
+                             // tile writes fp32 partial sums to the split workspace (c_off then points there)
+    int reserved;
     int64_t b_off;           // element offset of the group's weight block
     int64_t c_off;           // element offset of the group's output block
 };
 
+// One small tail tile row whose reduction was split into `parts` ranges: the partial sums of part s and local row r
+// are row (pair0 + s) * kSplitRows + r of the split workspace ([.., cols] fp32).
+struct SplitTail {
+    int row_begin, rows;
+    int pair0, parts;
+};
+constexpr int kSplitRows = 128;          // rows reserved per (tail, part) pair: the largest small tile
+constexpr int kMaxSplit = 4;             // most parts a reduction is split into
+constexpr int kSplitCus = 256;           // a launch's split parts never number more than this (one round of MI355X's CUs)
+constexpr int kSplitMinRed = 2048;       // shortest reduction range worth a part of its own
+
 struct TileTable {
     int slots_per_xcd;       // sum of the entries' shares
     int num_entries;
-    int pad[6];
+    int num_split_tails;     // tail tile rows whose reduction was split (entries of the SplitTail array in use)
+    int pad[5];
     int zeros[8];            // always zero: source of out-of-range operand chunks (holds an aligned 16-byte block)
     int begins[16];          // tile_begin of the first 16 entries (INT_MAX past the last): one load finds the entry
     GroupEntry entries[1];
@@ -55,6 +70,8 @@ struct GmmArgs {
     int64_t fc1_stride_row;
     float *partials;           // [rows, partials_per_row] row sums of dact * silu(gate) * up per 64 columns, or NULL
     int partials_per_row;
+    // split tail tiles only (OUT_SAME): fp32 partial sums, rows of `cols` floats
+    float *split_ws;
 };
 
 struct TileCoord {

@@ -754,9 +754,21 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
     const TileCoord tc = locate_tile(p.table);
     if (!tc.valid) return;
     MS_TRACE(2);
-    if (tc.tile_rows == 256) gmm16_tile<DT, A_RED, B_RED, OUT, 256>(p, tc, lds);
-    else if (tc.tile_rows == 128) gmm16_tile<DT, A_RED, B_RED, OUT, 128>(p, tc, lds);
-    else gmm16_tile<DT, A_RED, B_RED, OUT, 64>(p, tc, lds);
+    if (tc.tile_rows == 256) {
+        gmm16_tile<DT, A_RED, B_RED, OUT, 256>(p, tc, lds);
+    } else if (OUT == OUT_SAME && A_RED && tc.e.split != 0) {
+        // one part of a small tail tile whose reduction is split: fp32 partial sums into the split workspace
+        // (rows of `cols` floats; the entry's c_off leads to this part's block)
+        GmmArgs q = p;
+        q.c = p.split_ws;
+        q.c_stride_row = p.cols;
+        if (tc.tile_rows == 128) gmm16_tile<DT, A_RED, B_RED, OUT_F32, 128>(q, tc, lds);
+        else gmm16_tile<DT, A_RED, B_RED, OUT_F32, 64>(q, tc, lds);
+    } else if (tc.tile_rows == 128) {
+        gmm16_tile<DT, A_RED, B_RED, OUT, 128>(p, tc, lds);
+    } else {
+        gmm16_tile<DT, A_RED, B_RED, OUT, 64>(p, tc, lds);
+    }
 #ifdef MS_TRACE_TILES
     if (threadIdx.x == 0) {
         unsigned hw_id, xcc_id;

@@ -53,7 +53,9 @@ def _gmm_launch(x, weight, group_list, group_type, group_list_type, out, accumul
     num_groups = group_list.numel()
     out_dtype = _lib.MS_FP32 if out.dtype == torch.float32 else dtype
     nbytes = ctypes.c_size_t(0)
-    _lib.check(lib.ms_gmm_workspace_size(num_groups, m, group_type, ctypes.byref(nbytes)), "ms_gmm_workspace_size")
+    _lib.check(lib.ms_gmm_workspace_size_split(num_groups, m, k, n, group_type, dtype, out_dtype,
+                                               1 if accumulate else 0, ctypes.byref(nbytes)),
+               "ms_gmm_workspace_size_split")
     ws = _lib.workspace(nbytes.value, dev)
     # kernel flavour by operand layout: NN (forward), NT (weight read transposed: dX), TN (dW)
     if group_type == 2:

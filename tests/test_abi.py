@@ -42,6 +42,23 @@ def test_workspace_size_and_validation_are_host_only():
     assert b"exceeds" in lib.ms_last_error()
     assert lib.ms_gmm_workspace_size(8, 8192, 0, ctypes.byref(n)) == 0 and n.value >= 8 * 40
     assert lib.ms_gmm_workspace_size(0, 8192, 0, ctypes.byref(n)) != 0
+    # the second query adds room for partial sums only where tail tiles may be split: split on rows, 16-bit output,
+    # few rounds of tiles over a long reduction
+    base, m2 = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert lib.ms_gmm_workspace_size(8, 8192, 0, ctypes.byref(base)) == 0
+    BF16, FP32 = 0, 2
+    assert lib.ms_gmm_workspace_size_split(8, 8192, 14336, 4096, 0, BF16, BF16, 0, ctypes.byref(m2)) == 0
+    assert base.value + (16 << 20) <= m2.value <= base.value + (32 << 20) + 4096       # fc2 forward of the Mixtral shape
+    for args in [(8, 8192, 4096, 28672, 0, BF16, BF16, 0),      # many rounds of tiles
+                 (8, 8192, 2048, 4096, 0, BF16, BF16, 0),       # short reduction
+                 (8, 8192, 14336, 4096, 2, BF16, BF16, 0),      # split on the reduction dim
+                 (8, 8192, 14336, 4096, 0, BF16, FP32, 1),      # fp32 accumulate form
+                 (8, 8192, 14336, 4096, 0, FP32, FP32, 0),      # fp32 operands
+                 (4, 600, 8192, 512, 0, BF16, BF16, 0)]:        # far less than a round of tiles
+        assert lib.ms_gmm_workspace_size_split(*args, ctypes.byref(m2)) == 0
+        assert lib.ms_gmm_workspace_size(args[0], args[1], args[4], ctypes.byref(base)) == 0
+        assert m2.value == base.value, args
+    assert lib.ms_gmm_workspace_size_split(0, 8192, 14336, 4096, 0, BF16, BF16, 0, ctypes.byref(m2)) != 0
     # bad arguments are rejected before anything is launched
     rc = lib.ms_gmm(None, None, 1, 1, None, 1, 1, 1, None, 1, None, 0, 1, 8, 16, 16, 16, 0, 0, 0, None, 0)
     assert rc != 0 and b"group_type" in lib.ms_last_error()

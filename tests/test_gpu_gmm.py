@@ -230,3 +230,84 @@ def test_linearity_at_mixtral_fc1_shape(device):
         g = int(torch.searchsorted(bounds, torch.tensor(r), right=True))
         ref = x1[r].float().cpu() @ w[g].float().cpu()
         assert rel_l2(y1[r], ref) <= 1e-2, r
+
+
+# Launches that end in a round of small tail tiles over a long reduction: 31 or 32 row tiles of 256 rows in front
+# (8 column panels: 248 / 256 tiles on 256 compute units), then the 64- / 128-row tails, whose reduction the larger
+# workspace lets the library cut into parts.
+SPLIT_CASES = [
+    # counts (sum 8192 + ...), k, n
+    ([2098, 2049, 2148, 1897], 4096, 2048),          # two parts per tail
+    ([2098, 2049, 2148, 1897], 8264, 2048),          # four parts, the last one shorter and not a multiple of 64
+    ([2048, 2049, 2048, 2048 + 120], 16384, 2048),   # complete last round of full tiles; 1- and 120-row tails
+]
+
+
+def _gmm_abi(x, w, counts_dev, n, split, out):
+    """ms_gmm through ctypes with the plain or the larger (tail-splitting) workspace."""
+    import ctypes
+    from mindspeed_amd import _lib
+    lib = _lib.load()
+    m, k = x.shape
+    E = counts_dev.numel()
+    dt = _lib.dtype_code(x.dtype, "x")
+    nb = ctypes.c_size_t(0)
+    if split:
+        _lib.check(lib.ms_gmm_workspace_size_split(E, m, k, n, 0, dt, dt, 0, ctypes.byref(nb)), "size")
+    else:
+        _lib.check(lib.ms_gmm_workspace_size(E, m, 0, ctypes.byref(nb)), "size")
+    ws = torch.empty(nb.value, dtype=torch.uint8, device=x.device)
+    _lib.check(lib.ms_gmm(_lib.stream_ptr(x.device), _lib.ptr(x), x.stride(0), x.stride(1), _lib.ptr(w), w.stride(0),
+                          w.stride(1), w.stride(2), _lib.ptr(out), n, _lib.ptr(counts_dev), 1, 0, E, m, k, n, dt, dt, 0,
+                          _lib.ptr(ws), ws.numel()), "ms_gmm")
+    torch.cuda.synchronize()
+    return nb.value
+
+
+@pytest.mark.parametrize("counts,K,N,transposed,dtype",
+                         [(c, k, n, t, torch.bfloat16) for c, k, n in SPLIT_CASES for t in (False, True)] +
+                         [(*SPLIT_CASES[0], False, torch.float16), (*SPLIT_CASES[0], True, torch.float16)])
+def test_split_tail_tiles(counts, K, N, transposed, dtype, device):
+    """Tail tiles computed in parts along the reduction: rows outside the tails are bit-equal to the unsplit launch,
+    the tail rows match the oracle (fp32 CPU evaluation of just those rows) as closely as the unsplit launch does,
+    and the Python surface (which asks for the larger workspace) returns the split result."""
+    say("split tails", counts, K, N, transposed, dtype)
+    gen = torch.Generator().manual_seed(7)
+    M, E = sum(counts), len(counts)
+    x = torch.randn(M, K, generator=gen).to(dtype).to(device)
+    if transposed:
+        w = (torch.randn(E, N, K, generator=gen) * 0.05).to(dtype).to(device).transpose(1, 2)
+    else:
+        w = (torch.randn(E, K, N, generator=gen) * 0.05).to(dtype).to(device)
+    cdev = torch.tensor(counts, dtype=torch.int64, device=device)
+    plain = torch.full((M, N), float("nan"), dtype=dtype, device=device)
+    split = torch.full((M, N), float("nan"), dtype=dtype, device=device)
+    small = _gmm_abi(x, w, cdev, N, False, plain)
+    large = _gmm_abi(x, w, cdev, N, True, split)
+    assert large > small + (1 << 20)
+    ends = np.cumsum(counts)
+    tail_rows = []
+    for c, end in zip(counts, ends):
+        rem = c - (c - 1) // 256 * 256
+        if rem <= 128:
+            tail_rows += list(range(end - rem, end))
+    tail = torch.zeros(M, dtype=torch.bool)
+    tail[tail_rows] = True
+    assert torch.equal(plain[~tail.to(device)], split[~tail.to(device)])
+    assert not torch.isnan(split.float()).any()
+    # a different summation order over thousands of values leaves rounding differences somewhere in the tail rows:
+    # the larger workspace did take the split path
+    assert not torch.equal(plain[tail.to(device)], split[tail.to(device)])
+    # oracle on the tail rows only, group by group
+    xc, wc = x.cpu(), w.cpu()
+    start = 0
+    for g, (c, end) in enumerate(zip(counts, ends)):
+        rows = [r for r in tail_rows if start <= r < end]
+        if rows:
+            want = O.grouped_matmul(xc[rows], [len(rows)], wc[g:g + 1]).float()
+            e_split, e_plain = rel_l2(split[rows].float().cpu(), want), rel_l2(plain[rows].float().cpu(), want)
+            say("  group", g, "rows", len(rows), "rel-L2 split / plain", e_split, e_plain)
+            assert e_split <= TOL[dtype] and e_split <= 1.5 * e_plain + 1e-4
+        start = end
+    got = ops.npu_gmm_v2(x, w, group_list=cdev, group_type=0)
+    assert torch.equal(got, split)
