@@ -777,6 +777,7 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
         long long *rec = g_tile_trace + (blockIdx.x % kTraceSlots) * 8;
         rec[0] = (static_cast<long long>(xcc_id & 0xf) << 32) | ((hw_id >> 8) & 0xff) | (1ll << 40);   // XCC, CU/SH/SE bits, "valid"
         rec[5] = wall_clock64();
+        rec[6] = tc.tile_rows;
     }
 #endif
 }

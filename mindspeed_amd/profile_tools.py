@@ -242,15 +242,20 @@ def cmd_power(args):
             time.sleep(1.0)
 
 
-def _products(dev, data, gen):
-    """fc1-shaped products of the Mixtral expert MLP: name -> (callable, flops)."""
+def _products(dev, data, gen, counts=None):
+    """fc1-shaped products of the Mixtral expert MLP: name -> (callable, flops).  counts: rows per expert (eight equal
+    groups by default)."""
     import torch
 
     from .ops.gmm import gmm_raw
 
     T, H, F, E = 8192, 4096, 14336, 8
     bf = torch.bfloat16
-    counts = torch.full((E,), T // E, dtype=torch.int64, device=dev)
+    if counts:
+        T, E = sum(counts), len(counts)
+        counts = torch.tensor(counts, dtype=torch.int64, device=dev)
+    else:
+        counts = torch.full((E,), T // E, dtype=torch.int64, device=dev)
 
     def operand(*shape):
         if data == "zeros":
@@ -292,12 +297,15 @@ def cmd_timeline(args):
     dev = torch.device("cuda", 0)
     gen = torch.Generator(device=dev).manual_seed(0)
     slots = 16384
-    print("Mixtral-shape fc1 products (8192 rows in 8 equal groups, hidden 4096, 2*ffn 28672, bf16), one launch each; "
-          "times in microseconds from a 100 MHz clock, averaged over the workgroups that held a tile")
+    counts = [int(c) for c in args.counts.split(",")] if args.counts else None
+    groups = f"{sum(counts)} rows in groups of {args.counts}" if counts else "8192 rows in 8 equal groups"
+    print(f"Mixtral-shape fc1 products ({groups}, hidden 4096, 2*ffn 28672, bf16), one launch each; "
+          "times in microseconds from a 100 MHz clock, averaged over the workgroups that held a tile"
+          + (" of the given height (rows)" if counts else ""))
     print(f"{'product':8s} {'operands':8s} {'tiles':>6s} {'find tile':>10s} {'first data':>11s} {'K loop':>9s} {'epilogue':>9s} "
           f"{'tile total':>11s} {'idle gap':>9s} {'launch span':>12s} {'MFMA share':>11s}")
     for data in args.data.split(","):
-        make, flops = _products(dev, data, gen)
+        make, flops = _products(dev, data, gen, counts)
         for mode in args.modes.split(","):
             fn = make(mode)
             for _ in range(3):
@@ -314,6 +322,13 @@ def cmd_timeline(args):
             if len(rec) == 0:
                 print(f"{mode:8s} {data:8s} no records")
                 continue
+            heights = sorted(set(int(h) for h in rec[:, 6]), reverse=True)
+            if len(heights) > 1:                       # ragged groups: the phases of each tile height by itself
+                for h in heights:
+                    sub = rec[rec[:, 6] == h]
+                    ush = lambda a, b: float((sub[:, a] - sub[:, b]).mean()) / 100.0     # noqa: E731
+                    print(f"{mode + ' ' + str(h):8s} {data:8s} {len(sub):6d} {ush(2, 1):10.2f} {ush(3, 2):11.2f} {ush(4, 3):9.2f} "
+                          f"{ush(5, 4):9.2f} {ush(5, 1):11.2f}", flush=True)
             us = lambda a, b: float((rec[:, a] - rec[:, b]).mean()) / 100.0     # noqa: E731
             gaps = []
             by_cu = {}
@@ -351,6 +366,7 @@ def main():
     tl = sub.add_parser("timeline")
     tl.add_argument("--modes", default="fwd1,dx1,dw1")
     tl.add_argument("--data", default="randn,zeros")
+    tl.add_argument("--counts", default="", help="comma-separated rows per expert instead of eight equal groups")
     args = ap.parse_args()
     {"traffic": cmd_traffic, "counters": cmd_counters, "power": cmd_power, "timeline": cmd_timeline}[args.cmd](args)
 
