@@ -94,21 +94,23 @@ int ms_moe_token_permute_grad(ms_stream_t stream, const void *grad_permuted_toke
  * (mindspeed/ops/csrc/cann/npu_moe_token_unpermute.cpp:95-122; Python surface
  * mindspeed/ops/npu_moe_token_unpermute.py:13-22):
  *   out[t] = sum_j probs[t,j] * permuted[row_id_map[t*topk+j]]
- * probs may be NULL (unweighted sum).  fp32 accumulation, one rounding. */
+ * probs may be NULL (unweighted sum); probs_dtype is their own element type: dtype, or MS_FP32
+ * (fp32 router probabilities beside 16-bit tokens are used unrounded).  fp32 accumulation, one
+ * rounding to the tokens' dtype. */
 int ms_moe_token_unpermute(ms_stream_t stream, const void *permuted_tokens,
-                           const int32_t *row_id_map, const void *probs, int64_t num_tokens,
-                           int64_t topk, int64_t hidden, int dtype, int64_t num_permuted_rows,
-                           void *unpermuted_tokens);
+                           const int32_t *row_id_map, const void *probs, int probs_dtype,
+                           int64_t num_tokens, int64_t topk, int64_t hidden, int dtype,
+                           int64_t num_permuted_rows, void *unpermuted_tokens);
 
 /* Token unpermute backward — stands in for aclnnMoeTokenUnpermuteGrad
  * (npu_moe_token_unpermute.cpp:124-148):
  *   grad_permuted[row_id_map[t*topk+j]] = probs[t,j] * grad_out[t]
  *   grad_probs[t,j] = <grad_out[t], permuted[row_id_map[t*topk+j]]>   (fp32 dot)
  * probs / grad_probs / permuted_tokens may be NULL together (then
- * grad_permuted[row] = grad_out[token of row]). */
+ * grad_permuted[row] = grad_out[token of row]).  probs and grad_probs share probs_dtype. */
 int ms_moe_token_unpermute_grad(ms_stream_t stream, const void *permuted_tokens,
                                 const void *grad_unpermuted_tokens, const int32_t *row_id_map,
-                                const void *probs, int64_t num_tokens, int64_t topk,
+                                const void *probs, int probs_dtype, int64_t num_tokens, int64_t topk,
                                 int64_t hidden, int dtype, int64_t num_permuted_rows,
                                 void *grad_permuted_tokens, void *grad_probs);
 

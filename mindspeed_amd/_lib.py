@@ -15,6 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # MINDSPEED_AMD_LIB names another build of the same library (to compare two builds on one machine)
 LIB_PATH = os.environ.get("MINDSPEED_AMD_LIB") or os.path.join(_HERE, "libmindspeed_amd.so")
 
+ABI_VERSION = 101                # what ms_version() of a matching build returns (argument lists below)
 MS_BF16, MS_FP16, MS_FP32 = 0, 1, 2
 MS_INT32, MS_INT64 = 0, 1
 MS_MAX_EXPERTS = 1024
@@ -34,8 +35,8 @@ _SIGNATURES = {
     "ms_moe_token_permute": [_c_void_p, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _int, _i64, _i64,
                              _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _size_t],
     "ms_moe_token_permute_grad": [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _int, _i64, _c_void_p],
-    "ms_moe_token_unpermute": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _int, _i64, _c_void_p],
-    "ms_moe_token_unpermute_grad": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _int,
+    "ms_moe_token_unpermute": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _int, _i64, _c_void_p],
+    "ms_moe_token_unpermute_grad": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _int,
                                     _i64, _c_void_p, _c_void_p],
     "ms_moe_routing_map_workspace_size": [_i64, _i64, _int, ctypes.POINTER(_size_t)],
     "ms_moe_routing_map_permute": [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _int, _i64, _int, _c_void_p,
@@ -85,6 +86,10 @@ def load():
                 f"{LIB_PATH} is missing: the HIP kernels are the only compute path of mindspeed_amd. "
                 "Build them with `python -m mindspeed_amd.build` (needs hipcc).")
         lib = ctypes.CDLL(LIB_PATH)
+        lib.ms_version.argtypes, lib.ms_version.restype = [], _int
+        if lib.ms_version() != ABI_VERSION:
+            raise RuntimeError(f"{LIB_PATH} reports ABI version {lib.ms_version()}, this package binds version "
+                               f"{ABI_VERSION}: rebuild it with `python -m mindspeed_amd.build`")
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(lib, name)
             fn.argtypes = argtypes

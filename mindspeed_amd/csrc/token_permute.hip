@@ -401,11 +401,11 @@ __global__ __launch_bounds__(256) void permute_rows_kernel(const VecT *__restric
 // threads of a token (a power of two, part of one wavefront) look at `lanes` slots at a time and place the
 // valid ones with a ballot.  Probability gradients of the other slots are zeroed here when `zero` is given.
 constexpr int kCompactMaxLocal = 2048;   // (token, slot) pairs of one workgroup that the lists hold
-template <typename DT>
+template <typename PT>
 __device__ __forceinline__ int compact_slots(const int32_t *__restrict__ row_id_map,
-                                             const typename DT::storage *__restrict__ probs, int t, int topk,
+                                             const typename PT::storage *__restrict__ probs, int t, int topk,
                                              int num_rows, int lane, int lanes, int *ld, float *lw, int *lj,
-                                             typename DT::storage *__restrict__ zero) {
+                                             typename PT::storage *__restrict__ zero) {
     const int wl = threadIdx.x & 63;
     const int group0 = wl - lane;
     const unsigned long long group = (lanes == 64 ? ~0ull : ((1ull << lanes) - 1ull)) << group0;
@@ -420,10 +420,10 @@ __device__ __forceinline__ int compact_slots(const int32_t *__restrict__ row_id_
         if (valid) {
             const int pos = count + __popcll(bal & below);
             ld[pos] = d;
-            lw[pos] = probs != nullptr ? DT::to_float(probs[flat]) : 1.f;
+            lw[pos] = probs != nullptr ? PT::to_float(probs[flat]) : 1.f;
             if (lj != nullptr) lj[pos] = j;
         } else if (zero != nullptr && j < topk) {
-            zero[flat] = DT::from_float(0.f);
+            zero[flat] = PT::from_float(0.f);
         }
         count += __popcll(bal);
     }
@@ -435,10 +435,10 @@ __device__ __forceinline__ int compact_slots(const int32_t *__restrict__ row_id_
 // VEC: elements per thread access (16 bytes worth, or 1 for the unaligned path).
 // Row ids and weights are read once per thread; per group of U output vectors the row loads of up to JB
 // slots are independent and issued together; accumulation is fp32 in registers, slot by slot, one rounding.
-template <typename DT, int VEC, int JB, int U, bool COMPACT>
+template <typename DT, typename PT, int VEC, int JB, int U, bool COMPACT>
 __global__ __launch_bounds__(256) void gather_combine_kernel(
     const typename DT::storage *__restrict__ rows, const int32_t *__restrict__ row_id_map,
-    const typename DT::storage *__restrict__ probs, typename DT::storage *__restrict__ out,
+    const typename PT::storage *__restrict__ probs, typename DT::storage *__restrict__ out,
     int num_tokens, int topk, int hidden, int num_rows, int lanes) {
     using S = typename DT::storage;
     extern __shared__ int lds[];   // COMPACT: row ids [rows_per_block][topk], then weights
@@ -450,7 +450,8 @@ __global__ __launch_bounds__(256) void gather_combine_kernel(
     int *ld = lds + local_row * topk;
     float *lw = reinterpret_cast<float *>(lds + (256 / lanes) * topk) + local_row * topk;
     int nslots = topk;
-    if constexpr (COMPACT) nslots = compact_slots<DT>(row_id_map, probs, t, topk, num_rows, lane, lanes, ld, lw, nullptr, nullptr);
+    if constexpr (COMPACT)
+        nslots = compact_slots<PT>(row_id_map, probs, t, topk, num_rows, lane, lanes, ld, lw, nullptr, nullptr);
     for (int c0 = lane; c0 < vecs; c0 += U * lanes) {
         float acc[U][VEC];
 #pragma unroll
@@ -468,7 +469,7 @@ __global__ __launch_bounds__(256) void gather_combine_kernel(
                 } else {
                     const int64_t flat = static_cast<int64_t>(t) * topk + j0 + j;
                     d[j] = j0 + j < topk ? row_id_map[flat] : num_rows;
-                    w[j] = (probs != nullptr && j0 + j < topk) ? DT::to_float(probs[flat]) : 1.f;
+                    w[j] = (probs != nullptr && j0 + j < topk) ? PT::to_float(probs[flat]) : 1.f;
                 }
             }
             S tmp[JB][U][VEC];
@@ -521,11 +522,11 @@ __global__ __launch_bounds__(256) void gather_combine_kernel(
 // `lanes` threads (a power of two, one wavefront at most) share a token, so the dot products are folded with
 // lane shuffles and the kernel has no barrier.  Per chunk of U vectors a thread reads dY once and has the
 // loads of up to JB slots' rows in flight together.
-template <typename DT, int VEC, int JB, int U, bool COMPACT>
+template <typename DT, typename PT, int VEC, int JB, int U, bool COMPACT>
 __global__ __launch_bounds__(256) void unpermute_grad_kernel(
     const typename DT::storage *__restrict__ permuted, const typename DT::storage *__restrict__ grad_out,
-    const int32_t *__restrict__ row_id_map, const typename DT::storage *__restrict__ probs,
-    typename DT::storage *__restrict__ grad_permuted, typename DT::storage *__restrict__ grad_probs,
+    const int32_t *__restrict__ row_id_map, const typename PT::storage *__restrict__ probs,
+    typename DT::storage *__restrict__ grad_permuted, typename PT::storage *__restrict__ grad_probs,
     int num_tokens, int topk, int hidden, int num_rows, int lanes) {
     using S = typename DT::storage;
     const int local_row = threadIdx.x / lanes;
@@ -541,7 +542,7 @@ __global__ __launch_bounds__(256) void unpermute_grad_kernel(
     int *lj = lds + 2 * (256 / lanes) * topk + local_row * topk;
     int nslots = topk;
     if constexpr (COMPACT)
-        nslots = compact_slots<DT>(row_id_map, probs, t, topk, num_rows, lane, lanes, ld, lw, lj, grad_probs);
+        nslots = compact_slots<PT>(row_id_map, probs, t, topk, num_rows, lane, lanes, ld, lw, lj, grad_probs);
     for (int j0 = 0; j0 < nslots; j0 += JB) {
         int d[JB];
         float w[JB], dot[JB];
@@ -553,7 +554,7 @@ __global__ __launch_bounds__(256) void unpermute_grad_kernel(
             } else {
                 const int64_t flat = static_cast<int64_t>(t) * topk + j0 + j;
                 d[j] = j0 + j < topk ? row_id_map[flat] : num_rows;          // ids outside [0, num_rows): dropped
-                w[j] = (probs != nullptr && j0 + j < topk) ? DT::to_float(probs[flat]) : 1.f;
+                w[j] = (probs != nullptr && j0 + j < topk) ? PT::to_float(probs[flat]) : 1.f;
             }
             dot[j] = 0.f;
         }
@@ -622,7 +623,7 @@ __global__ __launch_bounds__(256) void unpermute_grad_kernel(
                 for (int dlt = lanes >> 1; dlt > 0; dlt >>= 1) s += __shfl_xor(s, dlt, 64);
                 if (lane == 0 && j0 + j < nslots) {
                     const int slot = COMPACT ? lj[j0 + j] : j0 + j;
-                    grad_probs[static_cast<int64_t>(t) * topk + slot] = DT::from_float(s);
+                    grad_probs[static_cast<int64_t>(t) * topk + slot] = PT::from_float(s);
                 }
             }
         }
@@ -1485,63 +1486,66 @@ int permute_fused_dispatch(hipStream_t stream, const SortPlan &p, const void *to
                                                 tpe_n, T, k, row_bytes);
 }
 
-template <typename DT>
+// PT: the probabilities' own type (the tokens' type, or fp32 beside 16-bit tokens)
+template <typename DT, typename PT>
 int launch_gather_combine(hipStream_t stream, const void *rows, const int32_t *map, const void *probs, void *out,
                           int64_t T, int64_t k, int64_t H, int64_t num_rows) {
     using S = typename DT::storage;
+    using PS = typename PT::storage;
     constexpr int VEC = 16 / sizeof(S);
     const bool vec_ok = (H % VEC == 0) && aligned16(rows) && aligned16(out);
     const int64_t vecs = vec_ok ? H / VEC : H;
     const RowLayout rl = row_layout(vecs);
     const unsigned blocks = static_cast<unsigned>(ceil_div(T, rl.rows_per_block));
 #define MS_GC_ARGS                                                                                                  \
-    static_cast<const S *>(rows), map, static_cast<const S *>(probs), static_cast<S *>(out), static_cast<int>(T),   \
+    static_cast<const S *>(rows), map, static_cast<const PS *>(probs), static_cast<S *>(out), static_cast<int>(T),  \
         static_cast<int>(k), static_cast<int>(H), static_cast<int>(num_rows), rl.lanes
     // many slots per token (the routing-map form has one per expert): list the valid ones first
     const bool compact = k > 8 && rl.rows_per_block * k <= kCompactMaxLocal;
     const size_t lds = compact ? static_cast<size_t>(2) * rl.rows_per_block * k * sizeof(int) : 0;
     if (!vec_ok && compact) {
-        hipLaunchKernelGGL((gather_combine_kernel<DT, 1, 8, 2, true>), dim3(blocks), dim3(256), lds, stream, MS_GC_ARGS);
+        hipLaunchKernelGGL((gather_combine_kernel<DT, PT, 1, 8, 2, true>), dim3(blocks), dim3(256), lds, stream, MS_GC_ARGS);
     } else if (!vec_ok) {
-        hipLaunchKernelGGL((gather_combine_kernel<DT, 1, 8, 2, false>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
+        hipLaunchKernelGGL((gather_combine_kernel<DT, PT, 1, 8, 2, false>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
     } else if (compact) {
-        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC, 8, 2, true>), dim3(blocks), dim3(256), lds, stream, MS_GC_ARGS);
+        hipLaunchKernelGGL((gather_combine_kernel<DT, PT, VEC, 8, 2, true>), dim3(blocks), dim3(256), lds, stream, MS_GC_ARGS);
     } else if (k <= 2) {
-        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC, 2, 4, false>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
+        hipLaunchKernelGGL((gather_combine_kernel<DT, PT, VEC, 2, 4, false>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
     } else {
-        hipLaunchKernelGGL((gather_combine_kernel<DT, VEC, 8, 2, false>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
+        hipLaunchKernelGGL((gather_combine_kernel<DT, PT, VEC, 8, 2, false>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
     }
 #undef MS_GC_ARGS
     MS_CHECK_LAUNCH("gather_combine_kernel");
     return MS_OK;
 }
 
-template <typename DT>
+template <typename DT, typename PT>
 int launch_unpermute_grad(hipStream_t stream, const void *permuted, const void *gy, const int32_t *map,
                           const void *probs, void *gperm, void *gprobs, int64_t T, int64_t k, int64_t H,
                           int64_t num_rows) {
     using S = typename DT::storage;
+    using PS = typename PT::storage;
     constexpr int VEC = 16 / sizeof(S);
     const bool vec_ok = (H % VEC == 0) && aligned16(gy) && aligned16(gperm) && (permuted == nullptr || aligned16(permuted));
     const int64_t vecs = vec_ok ? H / VEC : H;
     const RowLayout rl = row_layout(vecs);
     const dim3 grid(static_cast<unsigned>(ceil_div(T, rl.rows_per_block)));
 #define MS_UG_ARGS                                                                                                   \
-    static_cast<const S *>(permuted), static_cast<const S *>(gy), map, static_cast<const S *>(probs),                \
-        static_cast<S *>(gperm), static_cast<S *>(gprobs), static_cast<int>(T), static_cast<int>(k),                 \
+    static_cast<const S *>(permuted), static_cast<const S *>(gy), map, static_cast<const PS *>(probs),               \
+        static_cast<S *>(gperm), static_cast<PS *>(gprobs), static_cast<int>(T), static_cast<int>(k),                \
         static_cast<int>(H), static_cast<int>(num_rows), rl.lanes
     const bool compact = k > 8 && rl.rows_per_block * k <= kCompactMaxLocal;
     const size_t lds = compact ? static_cast<size_t>(3) * rl.rows_per_block * k * sizeof(int) : 0;
     if (!vec_ok && compact) {
-        hipLaunchKernelGGL((unpermute_grad_kernel<DT, 1, 4, 4, true>), grid, dim3(256), lds, stream, MS_UG_ARGS);
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, PT, 1, 4, 4, true>), grid, dim3(256), lds, stream, MS_UG_ARGS);
     } else if (!vec_ok) {
-        hipLaunchKernelGGL((unpermute_grad_kernel<DT, 1, 4, 4, false>), grid, dim3(256), 0, stream, MS_UG_ARGS);
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, PT, 1, 4, 4, false>), grid, dim3(256), 0, stream, MS_UG_ARGS);
     } else if (compact) {
-        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC, 4, 2, true>), grid, dim3(256), lds, stream, MS_UG_ARGS);
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, PT, VEC, 4, 2, true>), grid, dim3(256), lds, stream, MS_UG_ARGS);
     } else if (k <= 2) {
-        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC, 2, 4, false>), grid, dim3(256), 0, stream, MS_UG_ARGS);
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, PT, VEC, 2, 4, false>), grid, dim3(256), 0, stream, MS_UG_ARGS);
     } else {
-        hipLaunchKernelGGL((unpermute_grad_kernel<DT, VEC, 4, 2, false>), grid, dim3(256), 0, stream, MS_UG_ARGS);
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, PT, VEC, 4, 2, false>), grid, dim3(256), 0, stream, MS_UG_ARGS);
     }
 #undef MS_UG_ARGS
     MS_CHECK_LAUNCH("unpermute_grad_kernel");
@@ -1641,18 +1645,25 @@ extern "C" int ms_moe_token_permute(ms_stream_t stream_, const void *tokens, con
 }
 
 extern "C" int ms_moe_token_unpermute(ms_stream_t stream_, const void *permuted, const int32_t *row_id_map,
-                                      const void *probs, int64_t T, int64_t k, int64_t H, int dtype,
+                                      const void *probs, int probs_dtype, int64_t T, int64_t k, int64_t H, int dtype,
                                       int64_t num_rows, void *out) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (int rc = check_common("ms_moe_token_unpermute", T, k, H, dtype)) return rc;
+    MS_REQUIRE(probs == nullptr || probs_dtype == dtype || probs_dtype == MS_FP32, MS_ERR_UNSUPPORTED,
+               "ms_moe_token_unpermute: probs dtype %d must be the tokens' dtype (%d) or fp32", probs_dtype, dtype);
+    const bool p32 = probs != nullptr && probs_dtype == MS_FP32;
     MS_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31), MS_ERR_INVALID_ARGUMENT, "ms_moe_token_unpermute: bad num_permuted_rows");
     if (T == 0) return MS_OK;
     MS_REQUIRE((permuted || num_rows == 0) && row_id_map && out, MS_ERR_INVALID_ARGUMENT,
                "ms_moe_token_unpermute: NULL tensor pointer");
     switch (dtype) {
-        case MS_BF16: return launch_gather_combine<BF16>(stream, permuted, row_id_map, probs, out, T, k, H, num_rows);
-        case MS_FP16: return launch_gather_combine<FP16>(stream, permuted, row_id_map, probs, out, T, k, H, num_rows);
-        default: return launch_gather_combine<FP32>(stream, permuted, row_id_map, probs, out, T, k, H, num_rows);
+        case MS_BF16:
+            return p32 ? launch_gather_combine<BF16, FP32>(stream, permuted, row_id_map, probs, out, T, k, H, num_rows)
+                       : launch_gather_combine<BF16, BF16>(stream, permuted, row_id_map, probs, out, T, k, H, num_rows);
+        case MS_FP16:
+            return p32 ? launch_gather_combine<FP16, FP32>(stream, permuted, row_id_map, probs, out, T, k, H, num_rows)
+                       : launch_gather_combine<FP16, FP16>(stream, permuted, row_id_map, probs, out, T, k, H, num_rows);
+        default: return launch_gather_combine<FP32, FP32>(stream, permuted, row_id_map, probs, out, T, k, H, num_rows);
     }
 }
 
@@ -1660,15 +1671,18 @@ extern "C" int ms_moe_token_permute_grad(ms_stream_t stream, const void *grad_pe
                                          int64_t T, int64_t k, int64_t H, int dtype, int64_t num_rows,
                                          void *grad_tokens) {
     // The backward of a row gather is the unweighted top-k gather-sum.
-    return ms_moe_token_unpermute(stream, grad_permuted, row_id_map, nullptr, T, k, H, dtype, num_rows, grad_tokens);
+    return ms_moe_token_unpermute(stream, grad_permuted, row_id_map, nullptr, dtype, T, k, H, dtype, num_rows, grad_tokens);
 }
 
 extern "C" int ms_moe_token_unpermute_grad(ms_stream_t stream_, const void *permuted, const void *grad_out,
-                                           const int32_t *row_id_map, const void *probs, int64_t T, int64_t k,
-                                           int64_t H, int dtype, int64_t num_rows, void *grad_permuted,
+                                           const int32_t *row_id_map, const void *probs, int probs_dtype, int64_t T,
+                                           int64_t k, int64_t H, int dtype, int64_t num_rows, void *grad_permuted,
                                            void *grad_probs) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (int rc = check_common("ms_moe_token_unpermute_grad", T, k, H, dtype)) return rc;
+    MS_REQUIRE(probs == nullptr || probs_dtype == dtype || probs_dtype == MS_FP32, MS_ERR_UNSUPPORTED,
+               "ms_moe_token_unpermute_grad: probs dtype %d must be the tokens' dtype (%d) or fp32", probs_dtype, dtype);
+    const bool p32 = probs != nullptr && probs_dtype == MS_FP32;
     MS_REQUIRE(num_rows >= 0 && num_rows <= T * k, MS_ERR_INVALID_ARGUMENT,
                "ms_moe_token_unpermute_grad: num_permuted_rows %lld outside [0, %lld]", (long long)num_rows,
                (long long)(T * k));
@@ -1680,9 +1694,12 @@ extern "C" int ms_moe_token_unpermute_grad(ms_stream_t stream_, const void *perm
     MS_REQUIRE(grad_out && row_id_map && (grad_permuted || num_rows == 0), MS_ERR_INVALID_ARGUMENT,
                "ms_moe_token_unpermute_grad: NULL tensor pointer");
     switch (dtype) {
-        case MS_BF16: return launch_unpermute_grad<BF16>(stream, permuted, grad_out, row_id_map, probs, grad_permuted, grad_probs, T, k, H, num_rows);
-        case MS_FP16: return launch_unpermute_grad<FP16>(stream, permuted, grad_out, row_id_map, probs, grad_permuted, grad_probs, T, k, H, num_rows);
-        default: return launch_unpermute_grad<FP32>(stream, permuted, grad_out, row_id_map, probs, grad_permuted, grad_probs, T, k, H, num_rows);
+#define MS_UG_CALL(DT_, PT_) \
+    launch_unpermute_grad<DT_, PT_>(stream, permuted, grad_out, row_id_map, probs, grad_permuted, grad_probs, T, k, H, num_rows)
+        case MS_BF16: return p32 ? MS_UG_CALL(BF16, FP32) : MS_UG_CALL(BF16, BF16);
+        case MS_FP16: return p32 ? MS_UG_CALL(FP16, FP32) : MS_UG_CALL(FP16, FP16);
+        default: return MS_UG_CALL(FP32, FP32);
+#undef MS_UG_CALL
     }
 }
 

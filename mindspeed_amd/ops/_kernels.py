@@ -151,15 +151,25 @@ _define("moe_token_permute_grad(Tensor grad_permuted, Tensor row_id_map, int num
         _permute_grad, lambda g, r, num_tokens, topk: g.new_empty((num_tokens, g.size(1))))
 
 
+def _kernel_probs(probs, token_dtype):
+    """The kernels take probabilities in the tokens' dtype or in fp32; any other pair (fp16 beside bf16, 16-bit beside
+    fp32 tokens) is widened to fp32 first, which is exact."""
+    if probs is None or probs.dtype in (token_dtype, torch.float32):
+        return probs
+    return probs.float()
+
+
 def _unpermute(permuted, row_id_map, probs, num_tokens, topk):
     lib = _lib.load()
     dev = permuted.device
     hidden = permuted.size(1)
+    probs = _kernel_probs(probs, permuted.dtype)
     out = torch.empty((num_tokens, hidden), dtype=permuted.dtype, device=dev)
     work = flop_counter.unpermute_bytes(num_tokens, topk, hidden, permuted.element_size(), permuted.size(0))
     with torch.cuda.device(dev), flop_counter.op("unpermute", work, "byte", dev):
         _lib.check(lib.ms_moe_token_unpermute(
-            _lib.stream_ptr(dev), _lib.ptr(permuted), _lib.ptr(row_id_map), _lib.ptr(probs), num_tokens, topk, hidden,
+            _lib.stream_ptr(dev), _lib.ptr(permuted), _lib.ptr(row_id_map), _lib.ptr(probs),
+            _lib.dtype_code(probs.dtype, "probs") if probs is not None else 0, num_tokens, topk, hidden,
             _lib.dtype_code(permuted.dtype, "permuted_tokens"), permuted.size(0), _lib.ptr(out)),
             "ms_moe_token_unpermute")
     return out
@@ -175,6 +185,8 @@ def _unpermute_grad(permuted, grad_out, row_id_map, probs, num_tokens, topk, num
     dev = grad_out.device
     hidden = grad_out.size(1)
     rows = num_rows
+    probs_dtype = probs.dtype if probs is not None else None
+    probs = _kernel_probs(probs, grad_out.dtype)
     grad_permuted = torch.empty((rows, hidden), dtype=grad_out.dtype, device=dev)
     grad_probs = torch.empty_like(probs) if probs is not None else torch.empty(0, dtype=grad_out.dtype, device=dev)
     mapped = min(rows, num_tokens * topk)
@@ -184,9 +196,12 @@ def _unpermute_grad(permuted, grad_out, row_id_map, probs, num_tokens, topk, num
     with torch.cuda.device(dev), flop_counter.op("unpermute_grad", work, "byte", dev):
         _lib.check(lib.ms_moe_token_unpermute_grad(
             _lib.stream_ptr(dev), _lib.ptr(permuted) if probs is not None else None, _lib.ptr(grad_out),
-            _lib.ptr(row_id_map), _lib.ptr(probs), num_tokens, topk, hidden,
+            _lib.ptr(row_id_map), _lib.ptr(probs), _lib.dtype_code(probs.dtype, "probs") if probs is not None else 0,
+            num_tokens, topk, hidden,
             _lib.dtype_code(grad_out.dtype, "unpermuted_tokens_grad"), mapped, _lib.ptr(grad_permuted),
             _lib.ptr(grad_probs) if probs is not None else None), "ms_moe_token_unpermute_grad")
+    if probs is not None and grad_probs.dtype != probs_dtype:
+        grad_probs = grad_probs.to(probs_dtype)
     return grad_permuted, grad_probs
 
 

@@ -205,8 +205,8 @@ class MoeUnpermuteMaskMap(torch.autograd.Function):
             if probs.shape != routing_map.shape:
                 raise RuntimeError(f"probs shape {tuple(probs.shape)} differs from routing_map shape "
                                    f"{tuple(routing_map.shape)}")
-            ctx.probs_dtype = probs.dtype
-            probs = probs.contiguous().to(permuted_tokens.dtype)
+            _lib.dtype_code(probs.dtype, "probs")
+            probs = probs.contiguous()          # used in their own dtype, e.g. fp32 beside bf16 tokens
         out = K.moe_token_unpermute(permuted_tokens, row_id_map, probs, num_tokens, num_experts)
         ctx.save_for_backward(permuted_tokens if probs is not None else None, row_id_map, probs)
         ctx.num_tokens, ctx.num_experts, ctx.num_rows, ctx.hidden = num_tokens, num_experts, num_rows, hidden
@@ -223,9 +223,7 @@ class MoeUnpermuteMaskMap(torch.autograd.Function):
         grad_permuted, grad_probs = K.moe_token_unpermute_grad(
             permuted_tokens if probs is not None else grad_out.new_empty(0), grad_out, row_id_map, probs,
             ctx.num_tokens, ctx.num_experts, ctx.num_rows)
-        if probs is not None and ctx.needs_input_grad[3]:
-            grad_probs = grad_probs.to(ctx.probs_dtype)
-        else:
+        if probs is None or not ctx.needs_input_grad[3]:
             grad_probs = None
         return grad_permuted, None, None, grad_probs, None, None
 

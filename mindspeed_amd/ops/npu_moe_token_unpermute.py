@@ -76,10 +76,11 @@ def npu_moe_token_unpermute(permuted_tokens: torch.Tensor, sorted_indices: torch
     """``out[t] = sum_j probs[t, j] * permuted_tokens[sorted_indices[t*topk+j]]``.
 
     ``sorted_indices`` is the int32 map returned by ``npu_moe_token_permute``;
-    ``topk`` is ``probs.size(1)`` (1 without probs).  fp32 accumulation, one
-    rounding.  ``restore_shape`` is accepted and ignored, as in the reference.
+    ``topk`` is ``probs.size(1)`` (1 without probs).  ``probs`` may have a dtype of
+    their own (fp32 router probabilities beside bf16 tokens): they are used
+    unrounded, and their gradient comes back in that dtype.  fp32 accumulation, one
+    rounding to the tokens' dtype.  ``restore_shape`` is accepted and ignored, as
+    in the reference.
     """
     _check_forward(permuted_tokens, sorted_indices, probs, padded_mode)
-    if probs is not None and probs.dtype != permuted_tokens.dtype:
-        probs = probs.to(permuted_tokens.dtype)
     return _MoeTokenUnpermute.apply(permuted_tokens, sorted_indices, probs)

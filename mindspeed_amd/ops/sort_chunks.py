@@ -5,7 +5,11 @@ moe_feature/overlap/moe_common.py:377-398 (fused form:
 mindspeed/lite/ops/triton/sort_chunks_by_idx.py:300-348):
 ``cat([split(input, split_sizes)[i] for i in sorted_idxs])``; the backward is
 the inverse row map.  ``split_sizes`` and ``sorted_idxs`` may be device
-tensors; nothing is read back to the host.
+tensors; nothing is read back to the host.  Given as host lists they are checked
+(``sorted_idxs`` a permutation, the sizes summing to the row count, which the
+reference's ``split`` / ``cat`` require too); device tensors cannot be checked
+without a read-back, so then the outputs and gradients are zero-initialised and
+rows that a partial map leaves out read as zeros.
 """
 from __future__ import annotations
 
@@ -24,18 +28,20 @@ def _as_i64(v, device):
 
 class _SortChunks(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, inp, split_sizes, sorted_idxs, probs):
+    def forward(ctx, inp, split_sizes, sorted_idxs, probs, checked):
         lib = _lib.load()
+        new = torch.empty_like if checked else torch.zeros_like
+        ctx.checked = checked
         _lib.require_device(inp, "input")
         if inp.dim() != 2:
             raise RuntimeError(f"input must be 2 dimensional, got {inp.dim()}-dimensional")
         inp = inp.contiguous()
         dev = inp.device
         rows, hidden = inp.shape
-        out = torch.empty_like(inp)
+        out = new(inp)
         row_map = torch.empty(rows, dtype=torch.int32, device=dev)
         p = probs.contiguous() if probs is not None else None
-        out_p = torch.empty_like(p) if p is not None else None
+        out_p = new(p) if p is not None else None
         if p is not None and p.numel() != rows:
             raise RuntimeError(f"probs has {p.numel()} entries, expected {rows}")
         with torch.cuda.device(dev):
@@ -56,32 +62,42 @@ class _SortChunks(torch.autograd.Function):
     def backward(ctx, grad_out, grad_probs, _grad_map):
         (row_map,) = ctx.saved_tensors
         if grad_out is None:
-            return None, None, None, None
+            return None, None, None, None, None
         lib = _lib.load()
+        new = torch.empty_like if ctx.checked else torch.zeros_like
         dev = grad_out.device
         g = grad_out.contiguous()
-        gi = torch.empty_like(g)
+        gi = new(g)
         with torch.cuda.device(dev):
             _lib.check(lib.ms_gather_rows(_lib.stream_ptr(dev), _lib.ptr(g), _lib.ptr(row_map), g.size(0), g.size(1),
                                           _lib.dtype_code(g.dtype, "grad"), 1, _lib.ptr(gi)), "ms_gather_rows")
         gp = None
         if ctx.has_probs and grad_probs is not None:
             gpc = grad_probs.contiguous()
-            gp = torch.empty_like(gpc)
+            gp = new(gpc)
             with torch.cuda.device(dev):
                 _lib.check(lib.ms_gather_rows(_lib.stream_ptr(dev), _lib.ptr(gpc), _lib.ptr(row_map), gpc.numel(), 1,
                                               _lib.dtype_code(gpc.dtype, "grad_probs"), 1, _lib.ptr(gp)),
                            "ms_gather_rows")
-        return gi, None, None, gp
+        return gi, None, None, gp, None
 
 
 def sort_chunks_by_idxs(input, split_sizes, sorted_idxs, probs=None, fused=True):
     """Returns ``(output, permuted_probs)`` like the reference hook."""
     del fused  # one code path
     dev = input.device
+    on_host = lambda v: not isinstance(v, torch.Tensor) or v.device.type == "cpu"     # noqa: E731
+    checked = on_host(split_sizes) and on_host(sorted_idxs)
+    if checked:
+        as_list = lambda v: [int(i) for i in (v.tolist() if isinstance(v, torch.Tensor) else v)]     # noqa: E731
+        sizes, order = as_list(split_sizes), as_list(sorted_idxs)
+        if sorted(order) != list(range(len(sizes))):
+            raise RuntimeError(f"sorted_idxs must be a permutation of 0..{len(sizes) - 1}, got {order}")
+        if min(sizes, default=0) < 0 or sum(sizes) != input.size(0):
+            raise RuntimeError(f"split_sizes {sizes} do not sum to the {input.size(0)} rows of input")
     split_sizes = _as_i64(split_sizes, dev)
     sorted_idxs = _as_i64(sorted_idxs, dev)
     if split_sizes.numel() != sorted_idxs.numel():
         raise RuntimeError("split_sizes and sorted_idxs must have the same length")
-    out, out_probs, _ = _SortChunks.apply(input, split_sizes, sorted_idxs, probs)
+    out, out_probs, _ = _SortChunks.apply(input, split_sizes, sorted_idxs, probs, checked)
     return out, out_probs

@@ -88,10 +88,10 @@ def measure(num_tokens=4096, hidden=4096, num_experts=8, topk=2, dtype=torch.bfl
             stream, P(b.x), P(rmap), T, E, H, code, rows, 0, P(b.perm), P(b.mask_map), P(b.mask_sorted), P(b.counts),
             P(b.ws_mask), b.ws_mask.numel()), T * H * elem + rows * H * elem + T * E * (1 + 4) + rows * 4),
         "unpermute": (lambda b: lib.ms_moe_token_unpermute(
-            stream, P(b.perm), P(b.row_id_map), P(probs), T, K, H, code, rows, P(b.out)),
+            stream, P(b.perm), P(b.row_id_map), P(probs), code, T, K, H, code, rows, P(b.out)),
             flop_counter.unpermute_bytes(T, K, H, elem)),
         "unpermute_grad": (lambda b: lib.ms_moe_token_unpermute_grad(
-            stream, P(b.perm), P(b.gy), P(b.row_id_map), P(probs), T, K, H, code, rows, P(b.gperm), P(b.gprobs)),
+            stream, P(b.perm), P(b.gy), P(b.row_id_map), P(probs), code, T, K, H, code, rows, P(b.gperm), P(b.gprobs)),
             flop_counter.unpermute_grad_bytes(T, K, H, elem)),
         "permute_grad": (lambda b: lib.ms_moe_token_permute_grad(
             stream, P(b.perm), P(b.row_id_map), T, K, H, code, rows, P(b.out)),
@@ -99,10 +99,10 @@ def measure(num_tokens=4096, hidden=4096, num_experts=8, topk=2, dtype=torch.bfl
         # the routing-map form of the three gathers: the same entry points with top-k = experts, a [tokens, experts]
         # row map whose unset entries hold an id past the last row, and [tokens, experts] probabilities
         "unpermute_mask": (lambda b: lib.ms_moe_token_unpermute(
-            stream, P(b.perm), P(b.mask_map), P(probs_mask), T, E, H, code, rows, P(b.out)),
+            stream, P(b.perm), P(b.mask_map), P(probs_mask), code, T, E, H, code, rows, P(b.out)),
             flop_counter.unpermute_bytes(T, K, H, elem) + T * (E - K) * (4 + elem)),
         "unpermute_mask_grad": (lambda b: lib.ms_moe_token_unpermute_grad(
-            stream, P(b.perm), P(b.gy), P(b.mask_map), P(probs_mask), T, E, H, code, rows, P(b.gperm),
+            stream, P(b.perm), P(b.gy), P(b.mask_map), P(probs_mask), code, T, E, H, code, rows, P(b.gperm),
             P(b.gprobs_mask)), flop_counter.unpermute_grad_bytes(T, K, H, elem) + T * (E - K) * (4 + 2 * elem)),
         "permute_mask_grad": (lambda b: lib.ms_moe_token_permute_grad(
             stream, P(b.perm), P(b.mask_map), T, E, H, code, rows, P(b.out)),

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in sorted(declared_symbols()):
         assert hasattr(lib, name), name
-    assert lib.ms_version() >= 100
+    assert lib.ms_version() == _lib.ABI_VERSION
 
 
 def test_workspace_size_and_validation_are_host_only():
@@ -66,7 +66,7 @@ def test_workspace_size_and_validation_are_host_only():
     assert rc != 0 and b"dtype" in lib.ms_last_error()
     rc = lib.ms_swiglu(None, None, None, 0, -1, 16, 0, None)
     assert rc != 0
-    rc = lib.ms_moe_token_unpermute(None, None, None, None, 4, 0, 16, 0, 8, None)
+    rc = lib.ms_moe_token_unpermute(None, None, None, None, 0, 4, 0, 16, 0, 8, None)
     assert rc != 0 and b"topk" in lib.ms_last_error()
     with pytest.raises(_lib.MindSpeedAmdError):
         _lib.check(rc, "ms_moe_token_unpermute")

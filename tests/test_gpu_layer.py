@@ -70,6 +70,39 @@ def test_sort_chunks(nchunks, rows, hidden, device):
     assert none is None and torch.equal(out2.cpu(), eo)
 
 
+def test_sort_chunks_partial_map_on_the_device(device):
+    """Sizes and order given as device tensors cannot be checked without a read-back: rows that a partial map leaves
+    out (sizes summing to less than the row count, a chunk named twice and another never) read as zeros, forward
+    and backward, instead of uninitialised memory."""
+    say("sort_chunks partial map")
+    gen = torch.Generator().manual_seed(5)
+    rows, hidden = 1000, 64
+    x = torch.randn(rows, hidden, generator=gen)
+    p = torch.rand(rows, generator=gen)
+    poison = torch.full((1 << 22,), float("nan"), device=device)       # whatever the allocator hands out next is NaN
+    del poison
+    # 1. the sizes cover 900 of the 1000 rows
+    sizes = torch.tensor([300, 100, 500]); order = torch.tensor([2, 0, 1])
+    xd = x.to(device).requires_grad_(True)
+    out, outp = ops.sort_chunks_by_idxs(xd, sizes.to(device), order.to(device), p.to(device))
+    want = torch.cat([x[400:900], x[0:300], x[300:400], torch.zeros(100, hidden)])
+    assert torch.equal(out.cpu(), want)
+    assert torch.equal(outp.cpu(), torch.cat([p[400:900], p[0:300], p[300:400], torch.zeros(100)]))
+    g = torch.randn(rows, hidden, generator=gen)
+    out.backward(g.to(device))
+    exp_g = torch.zeros(rows, hidden)
+    exp_g[400:900], exp_g[0:300], exp_g[300:400] = g[0:500], g[500:800], g[800:900]
+    assert torch.equal(xd.grad.cpu(), exp_g)
+    # 2. chunk 0 named twice, chunk 1 never: 600 output rows are written, the input rows of chunk 1 get no gradient
+    sizes = torch.tensor([300, 700]); order = torch.tensor([0, 0])
+    xd = x.to(device).requires_grad_(True)
+    out, _ = ops.sort_chunks_by_idxs(xd, sizes.to(device), order.to(device))
+    assert torch.equal(out.cpu(), torch.cat([x[0:300], x[0:300], torch.zeros(400, hidden)]))
+    out.backward(g.to(device))
+    got = xd.grad.cpu()
+    assert not torch.isnan(got).any() and torch.equal(got[300:], torch.zeros(700, hidden))
+
+
 @pytest.mark.parametrize("dtype,pdt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float32),
                                        (torch.float32, torch.float32)])
 @pytest.mark.parametrize("nchunks,rows,hidden", [(64, 8192, 512), (1500, 6000, 24), (2600, 40000, 8), (7, 300, 13)])

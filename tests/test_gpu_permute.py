@@ -176,6 +176,42 @@ def test_unpermute_forward_backward(T, k, E, H, dtype, num_out, device):
         assert torch.equal(back.cpu(), tokens)
 
 
+@pytest.mark.parametrize("tdtype,pdtype", [(torch.bfloat16, torch.float32), (torch.float16, torch.float32),
+                                           (torch.float32, torch.bfloat16)])
+def test_unpermute_probs_keep_their_own_dtype(tdtype, pdtype, device):
+    """Probabilities of another dtype than the tokens are used unrounded (the torch path multiplies bf16 tokens by
+    fp32 probabilities in fp32, mindspeed/core/transformer/moe/moe_utils.py:236-238), and their gradient is an fp32
+    dot product stored in the probabilities' dtype."""
+    say("unpermute mixed dtypes", tdtype, pdtype)
+    T, k, E, H = 256, 2, 8, 512
+    _, idx = routing(T, k, E, seed=3)
+    exp_map = O.fused_permute(torch.zeros(T, 1), idx, None)[1]
+    if pdtype == torch.float32:
+        # 1024 * (0.5 + 2^-11) - 1024 * 0.5 = 0.5 exactly; with the probabilities rounded to 16 bits first it is 0
+        x = torch.empty(T * k, H)
+        x[exp_map.long()] = torch.tensor([1024.0, -1024.0]).repeat(T)[:, None].expand(T * k, H)
+        probs = torch.tensor([0.5 + 2.0 ** -11, 0.5]).repeat(T, 1)
+        out = ops.npu_moe_token_unpermute(x.to(tdtype).to(device), exp_map.to(device), probs.to(device))
+        assert out.dtype == tdtype
+        assert torch.equal(out.float().cpu(), torch.full((T, H), 0.5))
+    gen = torch.Generator().manual_seed(11)
+    x = torch.randn(T * k, H, generator=gen).to(tdtype)
+    gy = torch.randn(T, H, generator=gen).to(tdtype)
+    probs = torch.rand(T, k, generator=gen).to(pdtype)
+    xd = x.to(device).requires_grad_(True)
+    pd = probs.to(device).requires_grad_(True)
+    out = ops.npu_moe_token_unpermute(xd, exp_map.to(device), pd)
+    out.backward(gy.to(device))
+    torch.cuda.synchronize()
+    assert out.dtype == tdtype and pd.grad.dtype == pdtype and xd.grad.dtype == tdtype
+    ref = O.fused_unpermute(x.double(), exp_map, probs.double())
+    gx, gp = O.unpermute_backward(gy.double(), x.double(), exp_map, probs.double())
+    assert rel_l2(out, ref) <= TOL[tdtype]
+    assert rel_l2(xd.grad, gx) <= TOL[tdtype]
+    # the dot products are exact products of the stored values summed in fp32: fp32 probabilities get them unrounded
+    assert rel_l2(pd.grad, gp) <= (1e-5 if pdtype == torch.float32 else TOL[pdtype])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_permute_backward_and_roundtrip(dtype, device):
     T, k, E, H = 640, 4, 16, 264

@@ -47,6 +47,20 @@ def test_no_cpu_fallback():
         ops.sort_chunks_by_idxs(x, [4, 4], [1, 0])
 
 
+def test_sort_chunks_checks_host_lists():
+    """Given on the host, the chunk sizes must sum to the row count and the order must be a permutation, as the
+    reference's split / cat require (moe_common.py:377-398)."""
+    x = torch.randn(8, 16, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="permutation"):
+        ops.sort_chunks_by_idxs(x, [4, 4], [0, 0])
+    with pytest.raises(RuntimeError, match="permutation"):
+        ops.sort_chunks_by_idxs(x, torch.tensor([4, 4]), torch.tensor([1, 2]))
+    with pytest.raises(RuntimeError, match="do not sum"):
+        ops.sort_chunks_by_idxs(x, [4, 3], [1, 0])
+    with pytest.raises(RuntimeError, match="do not sum"):
+        ops.sort_chunks_by_idxs(x, [9, -1], [1, 0])
+
+
 def test_permute_argument_checks():
     x = torch.randn(8, 16, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="padded_mode"):
