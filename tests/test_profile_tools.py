@@ -83,3 +83,17 @@ def test_tile_timeline_on_the_diagnostic_build():
     find, first, loop, epilogue, total = (float(v) for v in line[3:8])
     assert 0 < find and 0 < first and 0 < loop and 0 < epilogue
     assert abs(find + first + loop + epilogue - total) < 0.05 * total
+
+
+def test_tracked_traffic_profile_belongs_to_these_sources():
+    """bench.py reports roofline.traffic only from a profile measured on the kernel sources as they are now; a
+    profile left behind by an older build would make it report null."""
+    path = os.path.join(ROOT, "profiles", "gmm_hbm_traffic.json")
+    data = json.loads(open(path).read())
+    assert data["build"] == build.source_hash(), \
+        "profiles/gmm_hbm_traffic.json was measured on other kernel sources: re-run the two rocprofv3 --pmc passes " \
+        "named in profiles/moe_layer_mixtral_hbm_traffic.txt and `python -m mindspeed_amd.profile_tools traffic --out` it"
+    sys.path.insert(0, ROOT)
+    import bench
+    for kernel in ("gmm_fwd", "gmm_dx", "gmm_dw"):
+        assert bench.measured_traffic("mixtral", kernel) == data["bytes_per_launch"]["mixtral"][kernel] > 1e9
