@@ -136,6 +136,7 @@ int ms_moe_token_unpermute_grad(ms_stream_t stream, const void *permuted_tokens,
  * non-routed tokens in ascending order, cut at capacity — the selection
  * routing_map.T.argsort(descending, stable)[:, :capacity] makes; tokens_per_expert = capacity.
  * tokens / permuted_tokens may be NULL to compute the maps only (unpermute needs them again).
+ * Permuted rows that no entry maps to (num_out_tokens above the number of set entries) are zeros.
  * The row maps plug into ms_moe_token_permute_grad / ms_moe_token_unpermute[_grad] with
  * topk = num_experts.
  *

@@ -1090,6 +1090,26 @@ __global__ __launch_bounds__(256) void routing_map_probs_grad_kernel(const int32
     grad_probs[i] = static_cast<unsigned>(r) < static_cast<unsigned>(num_rows) ? grad_permuted_probs[r] : S(0);
 }
 
+// Permuted rows [first, num_rows) that no map entry leads to (the caller's row count exceeds the number of set
+// entries) are written as zeros, shared out over the workgroups of the launch.
+template <typename VecT>
+__device__ __forceinline__ void zero_unmapped_rows(VecT *__restrict__ permuted, int first, int num_rows, int vecs_per_row) {
+    for (int r = first + blockIdx.x; r < num_rows; r += gridDim.x) {
+        VecT *dst = permuted + static_cast<int64_t>(r) * vecs_per_row;
+        for (int c = threadIdx.x; c < vecs_per_row; c += blockDim.x) dst[c] = VecT{};
+    }
+}
+
+// The same for the sort-based path, which marks those rows in sorted_flat: one workgroup per 4 rows.
+template <typename VecT>
+__global__ __launch_bounds__(256) void zero_marked_rows_kernel(const int32_t *__restrict__ sorted_flat, int num_rows,
+                                                               int vecs_per_row, VecT *__restrict__ permuted) {
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= num_rows || sorted_flat[r] >= 0) return;
+    VecT *dst = permuted + static_cast<int64_t>(r) * vecs_per_row;
+    for (int c = threadIdx.x & 63; c < vecs_per_row; c += 64) dst[c] = VecT{};
+}
+
 // Mask mode, rows laid out and moved in one launch (no drop-and-pad, experts a power of two up to 16, so that
 // a 16-byte vector of the map holds whole tokens and byte position b of a vector always belongs to expert
 // b % E; maps up to kFusedMapMax entries).  Same scheme as permute_fused_kernel: every workgroup counts, per
@@ -1162,10 +1182,12 @@ __global__ __launch_bounds__(1024) void routing_map_fused_kernel(
         base[tid] = first + sums[tid];
         if (blockIdx.x == 0 && tokens_per_expert != nullptr) tokens_per_expert[tid] = sums[tid] + sums[16 + tid];
     }
-    if (blockIdx.x == 0) {   // rows that nothing maps to (only if the caller's row count exceeds the set entries)
+    {   // rows that nothing maps to (only if the caller's row count exceeds the set entries)
         int nnz = 0;
         for (int e = 0; e < E; ++e) nnz += sums[e] + sums[16 + e];
-        for (int r = nnz + tid; r < num_rows; r += nthreads) sorted_flat[r] = -1;
+        if (blockIdx.x == 0)
+            for (int r = nnz + tid; r < num_rows; r += nthreads) sorted_flat[r] = -1;
+        if (tokens != nullptr) zero_unmapped_rows(permuted, nnz, num_rows, vecs_per_row);
     }
     __syncthreads();
     // Own entries in flat order, 64 at a time: lane l always sees expert l % E (E divides 64).  An entry's row
@@ -1284,6 +1306,7 @@ __global__ __launch_bounds__(1024) void routing_map_ranked_kernel(
     }
     if (blockIdx.x == 0)   // rows that nothing maps to (only if the caller's row count exceeds the set entries)
         for (int r = carry + tid; r < num_rows; r += nthreads) sorted_flat[r] = -1;
+    if (tokens != nullptr) zero_unmapped_rows(permuted, carry, num_rows, vecs_per_row);
     for (int e = tid; e < E; e += nthreads) {
         int next = first[e] + pre[e] + cnt[e];
         for (int lt = 0; lt < t1 - t0; ++lt) {
@@ -1863,10 +1886,26 @@ extern "C" int ms_moe_routing_map_permute(ms_stream_t stream_, const void *token
     MS_CHECK_LAUNCH("routing_map_rows_kernel");
     if (tokens == nullptr || num_rows == 0) return MS_OK;
     const int64_t row_bytes = H * dtype_size(dtype);
-    if (row_bytes % 16 == 0 && aligned16(tokens) && aligned16(permuted))
-        return launch_permute_rows<v16>(stream, tokens, permuted, row_id_map, T, E, row_bytes, num_rows);
-    if (dtype == MS_FP32) return launch_permute_rows<uint32_t>(stream, tokens, permuted, row_id_map, T, E, row_bytes, num_rows);
-    return launch_permute_rows<uint16_t>(stream, tokens, permuted, row_id_map, T, E, row_bytes, num_rows);
+    // rows that no entry maps to (never in drop-and-pad mode, which fills every expert's block) are zeroed
+    const dim3 zgrid(static_cast<unsigned>(ceil_div(num_rows, 4)));
+    if (row_bytes % 16 == 0 && aligned16(tokens) && aligned16(permuted)) {
+        if (int rc = launch_permute_rows<v16>(stream, tokens, permuted, row_id_map, T, E, row_bytes, num_rows)) return rc;
+        if (!drop_and_pad)
+            hipLaunchKernelGGL(zero_marked_rows_kernel<v16>, zgrid, dim3(256), 0, stream, sorted_flat, static_cast<int>(num_rows),
+                               static_cast<int>(row_bytes / 16), static_cast<v16 *>(permuted));
+    } else if (dtype == MS_FP32) {
+        if (int rc = launch_permute_rows<uint32_t>(stream, tokens, permuted, row_id_map, T, E, row_bytes, num_rows)) return rc;
+        if (!drop_and_pad)
+            hipLaunchKernelGGL(zero_marked_rows_kernel<uint32_t>, zgrid, dim3(256), 0, stream, sorted_flat,
+                               static_cast<int>(num_rows), static_cast<int>(row_bytes / 4), static_cast<uint32_t *>(permuted));
+    } else {
+        if (int rc = launch_permute_rows<uint16_t>(stream, tokens, permuted, row_id_map, T, E, row_bytes, num_rows)) return rc;
+        if (!drop_and_pad)
+            hipLaunchKernelGGL(zero_marked_rows_kernel<uint16_t>, zgrid, dim3(256), 0, stream, sorted_flat,
+                               static_cast<int>(num_rows), static_cast<int>(row_bytes / 2), static_cast<uint16_t *>(permuted));
+    }
+    if (!drop_and_pad) MS_CHECK_LAUNCH("zero_marked_rows_kernel");
+    return MS_OK;
 }
 
 extern "C" int ms_moe_routing_map_probs(ms_stream_t stream_, const int32_t *sorted_flat, int64_t num_rows, int64_t E,

@@ -208,6 +208,31 @@ def test_no_entry_set(T, E, device):
     assert back.numel() == 0
 
 
+@pytest.mark.parametrize("T,E,k,H,dtype", [
+    (300, 8, 2, 256, torch.bfloat16),      # experts a power of two: one launch
+    (300, 6, 2, 264, torch.float32),       # any expert count: two launches
+    (257, 5, 3, 70, torch.float16),        # odd hidden: element path
+    (300, 900, 2, 32, torch.bfloat16),     # many experts: the sort-based path
+])
+def test_more_rows_than_set_entries(T, E, k, H, dtype, device):
+    """A row count above the number of set mask entries (no read-back of the count): the rows that nothing maps to
+    come back as zeros, their probabilities as zeros, and everything in front of them as usual."""
+    say("routing-map over-provisioned rows", T, E, k, H, dtype)
+    rmap, probs = make_map(T, E, k, seed=T + E)
+    tokens = torch.randn(T, H, generator=torch.Generator().manual_seed(1)).to(dtype)
+    nnz = int(rmap.sum())
+    extra = 77
+    poison = torch.full((1 << 22,), float("nan"), device=device)       # whatever the allocator hands out next is NaN
+    del poison
+    perm, pp, sidx = M.permute(tokens.to(device), rmap.to(device), probs.to(dtype).to(device), num_out_tokens=nnz + extra,
+                               fused=True)
+    o_perm, o_pp, o_sidx = O.permute_routing_map(tokens, rmap, probs.to(dtype))
+    assert perm.shape == (nnz + extra, H)
+    assert torch.equal(perm[:nnz].cpu(), o_perm) and torch.equal(pp[:nnz].cpu(), o_pp)
+    assert torch.equal(perm[nnz:].cpu(), torch.zeros(extra, H, dtype=dtype))
+    assert torch.equal(pp[nnz:].cpu(), torch.zeros(extra, dtype=dtype))
+
+
 def test_argument_checks(device):
     tokens = torch.randn(4, 8, device=device)
     rmap = torch.ones(4, 2, dtype=torch.bool, device=device)
