@@ -292,9 +292,8 @@ def main():
                    "gemm_tflop_per_step": round(18.0 * cfg["T"] * cfg["K"] * cfg["H"] * cfg["F"] / 1e12, 3)},
         "roofline": roofline,
         "kernels": kernels,
-        "kernels_note": "single launches inside the layer step, each between two events on its stream (the two "
-                        "weight-gradient products then run after, not beside, the dX products); an empty bracket "
-                        f"reads {empty_bracket_ms * 1e3:.1f} us on this box",
+        "kernels_note": "single launches inside the layer step, each between two events on its stream; an empty "
+                        f"bracket reads {empty_bracket_ms * 1e3:.1f} us on this box",
     }
     if args.copy_calibration:
         from mindspeed_amd import _lib
