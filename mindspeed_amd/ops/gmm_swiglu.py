@@ -153,10 +153,10 @@ class GroupedMLPFunction(torch.autograd.Function):
     backward  ``dact = dy @ w2^T``; ``d_fc1, d_probs = SwiGLU backward on the saved fc1``;
               ``dW2 = act^T dy``; ``dx = d_fc1 @ w1^T``; ``dW1 = x^T d_fc1``
 
-    One node instead of three keeps a second stream busy from start to end of the backward pass: dW2 runs
-    beside dX2 and the SwiGLU backward, dW1 beside dX1, with one join at the very end (measured on the
-    Mixtral shape this is no faster than three nodes that each overlap their own dW: the step is limited by
-    board power, not by idle units).
+    With ``MINDSPEED_AMD_OVERLAP_WGRAD=1`` one node instead of three keeps a second stream busy from start to end
+    of the backward pass: dW2 runs beside dX2 and the SwiGLU backward, dW1 beside dX1, with one join at the very
+    end (measured on the Mixtral shape this is no faster than three nodes that each overlap their own dW, nor than
+    no overlap at all: the step is limited by board power, not by idle units).
     ``fused_kernels``: the activation comes out of the first matmul's epilogue and its backward rides on the
     epilogue of the dX2 product (16-bit, vector-access layout only); otherwise one kernel per op, any dtype.
     ``recompute_activation``: ``act`` is not kept; backward rebuilds it from ``fc1`` for dW2.

@@ -1,5 +1,5 @@
-"""GPU: the whole single-rank expert layer (forward and backward, including the weight-gradient products on
-their second stream) recorded into a HIP graph and replayed.  Every replay, with eager work of the same ops and
+"""GPU: the whole single-rank expert layer (forward and backward; with and without the weight-gradient products
+on a second stream) recorded into a HIP graph and replayed.  Every replay, with eager work of the same ops and
 synchronisations in between, must reproduce the eager result bit for bit: the C ABI only launches kernels on
 the caller's stream (no allocation, no synchronisation, no memset node), which is what makes it capturable."""
 import pytest
@@ -36,10 +36,13 @@ def layer_step(x, idx, probs, w1, w2, gy, fuse):
     return (out,) + tuple(grads)
 
 
+@pytest.mark.parametrize("overlap", [False, True])
 @pytest.mark.parametrize("fuse", [False, True])
 @pytest.mark.parametrize("T,H,E,K,F", [(512, 256, 8, 2, 512), (300, 128, 6, 3, 200)])
-def test_layer_graph_replays_match_eager(T, H, E, K, F, fuse, device):
-    say("graph case", T, H, E, K, F, fuse)
+def test_layer_graph_replays_match_eager(T, H, E, K, F, fuse, overlap, device, monkeypatch):
+    say("graph case", T, H, E, K, F, fuse, overlap)
+    import mindspeed_amd.ops.gmm as gmm_ops
+    monkeypatch.setattr(gmm_ops, "OVERLAP_WGRAD", overlap)     # weight gradients beside dX on a second stream, or after
     dtype = torch.bfloat16
     a = make_inputs(T, H, E, K, F, dtype, device, seed=1)
     b = make_inputs(T, H, E, K, F, dtype, device, seed=2)

@@ -195,3 +195,30 @@ def test_mixtral_shape_sampled_tokens(device):
             a = (torch.nn.functional.silu(h[:F]) * h[F:]).to(torch.bfloat16).float()
             ref += p[t, j].float().cpu() * (a @ w2[e].float()).to(torch.bfloat16).float().cpu()
         assert rel_l2(out[t], ref) <= 1e-2, t
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+def test_weight_gradients_beside_dx_give_identical_results(fuse, device, monkeypatch):
+    """The optional second stream for the weight-gradient products (MINDSPEED_AMD_OVERLAP_WGRAD=1) changes when the
+    kernels run, not what they compute: every output and gradient of the layer is bit-equal to the default order."""
+    say("layer with and without the dX / dW overlap", fuse)
+    import mindspeed_amd.ops.gmm as gmm_ops
+    gen = torch.Generator().manual_seed(3)
+    T, H, E, K, F = 1500, 512, 8, 2, 768
+    x = torch.randn(T, H, generator=gen).to(torch.bfloat16).to(device)
+    probs, idx = torch.topk(torch.softmax(torch.randn(T, E, generator=gen), dim=-1), K, dim=-1)
+    probs, idx = probs.to(torch.bfloat16).to(device), idx.to(device)
+    w1 = (torch.randn(E, H, 2 * F, generator=gen) * 0.05).to(torch.bfloat16).to(device)
+    w2 = (torch.randn(E, F, H, generator=gen) * 0.05).to(torch.bfloat16).to(device)
+    gy = torch.randn(T, H, generator=gen).to(torch.bfloat16).to(device)
+    results = []
+    for overlap in (False, True, False):
+        monkeypatch.setattr(gmm_ops, "OVERLAP_WGRAD", overlap)
+        leaves = [t.detach().clone().requires_grad_(True) for t in (x, probs, w1, w2)]
+        out = dispatch_mlp_combine(leaves[0], idx, leaves[1], (leaves[2], leaves[3]), fuse_activation=fuse)
+        grads = torch.autograd.grad(out, leaves, gy)
+        torch.cuda.synchronize()
+        results.append((out,) + tuple(grads))
+    for other in results[1:]:
+        for a, b in zip(results[0], other):
+            assert torch.equal(a, b)
