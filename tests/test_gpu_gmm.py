@@ -311,3 +311,31 @@ def test_split_tail_tiles(counts, K, N, transposed, dtype, device):
         start = end
     got = ops.npu_gmm_v2(x, w, group_list=cdev, group_type=0)
     assert torch.equal(got, split)
+
+
+def test_split_tail_tiles_with_rows_past_the_last_offset(device):
+    """The tail split next to the zero-fill of rows that no group covers: those rows are zeros in both launches, the
+    rest matches as in test_split_tail_tiles."""
+    say("split tails + rows past the last offset")
+    counts, K, N, extra = [2098, 2049, 2148, 1897], 4096, 2048, 300
+    gen = torch.Generator().manual_seed(9)
+    M = sum(counts) + extra
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16).to(device)
+    w = (torch.randn(len(counts), K, N, generator=gen) * 0.05).to(torch.bfloat16).to(device)
+    cdev = torch.tensor(counts, dtype=torch.int64, device=device)
+    plain = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=device)
+    split = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=device)
+    _gmm_abi(x, w, cdev, N, False, plain)
+    _gmm_abi(x, w, cdev, N, True, split)
+    covered = sum(counts)
+    assert torch.equal(split[covered:], torch.zeros(extra, N, dtype=torch.bfloat16, device=device))
+    assert torch.equal(plain[covered:], split[covered:])
+    assert not torch.isnan(split.float()).any()
+    assert rel_l2(split[:covered].float().cpu(), plain[:covered].float().cpu()) <= 2e-3
+    full = torch.ones(M, dtype=torch.bool)
+    for c, end in zip(counts, np.cumsum(counts)):
+        rem = c - (c - 1) // 256 * 256
+        if rem <= 128:
+            full[end - rem:end] = False
+    full[covered:] = False
+    assert torch.equal(plain[full.to(device)], split[full.to(device)])
