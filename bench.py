@@ -63,18 +63,18 @@ def measured_traffic(workload, kernel):
     return data.get("bytes_per_launch", {}).get(workload, {}).get(kernel)
 
 
-def _cpu_layer_once(cfg, sample):
+def _cpu_layer_once(cfg, sample, dtype=torch.float32):
     from oracle import moe_oracle as O
 
     T, H, E, K, F = cfg["T"], cfg["H"], cfg["E"], cfg["K"], cfg["F"]
     sub = dict(cfg, T=sample)
     gen = torch.Generator().manual_seed(0)
-    x = torch.randn(sample, H, generator=gen).requires_grad_(True)
-    w1 = (torch.randn(E, H, 2 * F, generator=gen) * 0.02).requires_grad_(True)
-    w2 = (torch.randn(E, F, H, generator=gen) * 0.02).requires_grad_(True)
-    gy = torch.randn(sample, H, generator=gen)
+    x = torch.randn(sample, H, generator=gen).to(dtype).requires_grad_(True)
+    w1 = (torch.randn(E, H, 2 * F, generator=gen) * 0.02).to(dtype).requires_grad_(True)
+    w2 = (torch.randn(E, F, H, generator=gen) * 0.02).to(dtype).requires_grad_(True)
+    gy = torch.randn(sample, H, generator=gen).to(dtype)
     p, idx = make_routing(sub, 0)
-    p = p.requires_grad_(True)
+    p = p.to(dtype).requires_grad_(True)
     t0 = time.perf_counter()
     out = O.moe_layer(x, idx, p, w1, w2)
     torch.autograd.grad(out, (x, p, w1, w2), gy)
@@ -108,7 +108,21 @@ def cpu_baseline(cfg, budget_s=12.0):
     one = min(sample, 64)
     dt1 = _cpu_layer_once(cfg, one)
     torch.set_num_threads(threads)
-    return {"value": round(sample / dt, 2), "unit": "tokens/s", "cores": threads, "kind": "port",
+    # the workload's own dtype (bf16 matmuls on the CPU are the slower ones: fp32 above is the fair CPU figure)
+    extra = {}
+    if cfg["dtype"] == "bf16":
+        nb = min(sample, 64)
+        dtb = _cpu_layer_once(cfg, nb, torch.bfloat16)
+        extra["bf16"] = {"value": round(nb / dtb, 2), "unit": "tokens/s", "cores": threads,
+                         "sample": f"{nb} tokens, one forward+backward in bf16 ({dtb:.1f} s)"}
+    # configs[0], the reference's CPU-runnable case, whole (no extrapolation): median of five runs
+    from mindspeed_amd.workloads import WORKLOADS
+    small = WORKLOADS["plumbing"]
+    _cpu_layer_once(small, small["T"])
+    runs = sorted(_cpu_layer_once(small, small["T"]) for _ in range(5))
+    extra["plumbing_config"] = {"value": round(small["T"] / runs[2], 1), "unit": "tokens/s", "cores": threads,
+                                "sample": f"{small['desc']}, forward+backward, median of 5 runs ({runs[2] * 1e3:.1f} ms)"}
+    return {"value": round(sample / dt, 2), "unit": "tokens/s", "cores": threads, "kind": "port", **extra,
             "sample": f"{sample} of {T} tokens (extrapolated: every expert still reads its whole fp32 weights for that "
                       f"few rows, which is pessimistic for the CPU), same layer shape, fp32, one forward+backward "
                       f"({dt:.1f} s) with torch {torch.__version__} on {threads} threads",
