@@ -343,9 +343,9 @@ def main():
             others = {}
             del x, p, idx
             torch.cuda.empty_cache()
-            for name in ("deepseek", "qwen"):
+            for name in ("deepseek", "qwen", "plumbing"):
                 ocfg = WORKLOADS[name]
-                ms, _, ok, _ = run_layer(ocfg, device, steps=10, warmup=10)
+                ms, _, ok, _ = run_layer(ocfg, device, steps=10 if name != "plumbing" else 50, warmup=10)
                 others[name] = {"workload": ocfg["desc"], "ms_per_step": round(ms, 4),
                                 "tokens_per_s": round(ocfg["T"] / (ms / 1e3), 1),
                                 "gemm_tflops": {k: ok[k]["tflops"] for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok},
