@@ -954,7 +954,9 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
         args.split_ws = split_ws;
         if (int rc = launch_gmm16_fast(stream, args, dtype, out, a_is_red, b_is_red, grid)) return rc;
         if (split_ws != nullptr) {
-            const dim3 rgrid(static_cast<unsigned>(num_groups), static_cast<unsigned>(ceil_div(n, 2048)), 16);
+            // at most kSplitCus / (2 parts x column tiles) tails are ever split in one launch
+            const int64_t max_tails = kSplitCus / (2 * num_col_tiles) < num_groups ? kSplitCus / (2 * num_col_tiles) : num_groups;
+            const dim3 rgrid(static_cast<unsigned>(max_tails), static_cast<unsigned>(ceil_div(n, 2048)), 16);
             if (dtype == MS_BF16)
                 hipLaunchKernelGGL(gmm_split_reduce_kernel<MS_BF16>, rgrid, dim3(256), 0, stream, table, split_records,
                                    split_ws, static_cast<uint16_t *>(y), y_stride_row, static_cast<int>(n));
