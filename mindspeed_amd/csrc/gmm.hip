@@ -773,7 +773,8 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
                     const int64_t *group_list, int group_list_type, int group_type, int64_t num_groups, int64_t m,
                     int64_t k, int64_t n, int dtype, int out_dtype, int accumulate, void *workspace,
                     size_t workspace_bytes, const WeightOffsets *weight_offsets, bool all_weights_aligned16,
-                    const SwigluOut *swiglu = nullptr, const SwigluGradIn *swiglu_grad = nullptr) {
+                    const SwigluOut *swiglu = nullptr, const SwigluGradIn *swiglu_grad = nullptr,
+                    bool allow_split = true) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED, "ms_gmm: bad dtype %d", dtype);
     MS_REQUIRE(out_dtype == dtype || out_dtype == MS_FP32, MS_ERR_UNSUPPORTED,
@@ -834,7 +835,7 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     // plain one the launch runs unsplit.
     SplitTail *split_records = nullptr;
     float *split_ws = nullptr;
-    if (swiglu == nullptr && swiglu_grad == nullptr &&
+    if (allow_split && swiglu == nullptr && swiglu_grad == nullptr &&
         may_split_tails(m, k, n, group_type, dtype, out_dtype, accumulate, num_cus) &&
         workspace_bytes >= split_ws_pos(num_groups) + split_ws_bytes(n) &&
         (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
@@ -1031,7 +1032,7 @@ extern "C" int ms_gmm_noalloc(ms_stream_t stream, const void *x, int64_t x_strid
     if (int rc = scratch_of_current_device(&table)) return rc;
     return gmm_impl(stream, x, x_stride0, x_stride1, weight, w_stride_group, w_stride0, w_stride1, y, y_stride_row,
                     group_list, group_list_type, group_type, num_groups, m, k, n, dtype, out_dtype, accumulate, table,
-                    kScratchBytes, nullptr, false);
+                    kScratchBytes, nullptr, false, nullptr, nullptr, /*allow_split=*/false);
 }
 
 extern "C" int ms_gmm_swiglu(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1, const void *weight,
