@@ -95,6 +95,10 @@ GMM_CASES = [
     # forward, 6 x 9 in the weight gradient; 11 row tiles x 17 column panels (4 + 4 + 3, 8 + 8 + 1) in the last one
     (3000, 1536, 2304, 2, "random"),
     (2600, 1280, 4352, 1, "equal"),
+    # a single row tile left over after the blocks of 4 joins the last block: 9 row tiles x 10 column panels in
+    # forward (4 + 5), 5 x 10 in the weight gradient (one block of 5), and a ragged pair of groups with 5 row tiles each
+    (2300, 1280, 2560, 1, "equal"),
+    (2100, 768, 1024, 2, "equal"),
 ]
 
 
