@@ -197,6 +197,11 @@ int ms_gmm_workspace_size(int64_t num_groups, int64_t m, int group_type, size_t 
  * the two differ by the rounding of the summation order in the rows of those tail tiles only. */
 int ms_gmm_workspace_size_split(int64_t num_groups, int64_t m, int64_t k, int64_t n, int group_type,
                                 int dtype, int out_dtype, int accumulate, size_t *bytes);
+/* Diagnostic, host only (no counterpart in the reference): which tile of a group of num_row_tiles x
+ * num_col_tiles output tiles the grouped-matmul kernels take as their index-th (blocks of 4 row tiles x 8
+ * column panels, chosen for L2 reuse).  Evaluates the function the kernels call, so a test can check that
+ * the order visits every tile exactly once. */
+int ms_gmm_tile_order(int num_row_tiles, int num_col_tiles, int index, int *row_tile, int *col_tile);
 int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1,
            const void *weight, int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1,
            void *y, int64_t y_stride_row, const int64_t *group_list, int group_list_type,

@@ -725,6 +725,16 @@ extern "C" int ms_gmm_workspace_size(int64_t num_groups, int64_t m, int group_ty
     return MS_OK;
 }
 
+// The tile order of the kernels, evaluated on the host (the same function the kernels call).
+extern "C" int ms_gmm_tile_order(int num_row_tiles, int num_col_tiles, int index, int *row_tile, int *col_tile) {
+    MS_REQUIRE(num_row_tiles >= 1 && num_col_tiles >= 1 && index >= 0 &&
+                   static_cast<int64_t>(index) < static_cast<int64_t>(num_row_tiles) * num_col_tiles &&
+                   static_cast<int64_t>(num_row_tiles) * num_col_tiles < (1ll << 30) && row_tile != nullptr && col_tile != nullptr,
+               MS_ERR_INVALID_ARGUMENT, "ms_gmm_tile_order: bad arguments");
+    tile_order(index, num_row_tiles, num_col_tiles, *row_tile, *col_tile);
+    return MS_OK;
+}
+
 extern "C" int ms_gmm_workspace_size_split(int64_t num_groups, int64_t m, int64_t k, int64_t n, int group_type, int dtype,
                                            int out_dtype, int accumulate, size_t *bytes) {
     if (int rc = ms_gmm_workspace_size(num_groups, m, group_type, bytes)) return rc;

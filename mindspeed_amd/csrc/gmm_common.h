@@ -81,6 +81,29 @@ struct TileCoord {
     bool valid;
 };
 
+// Tile order inside a group of R row tiles x C column panels: the r-th tile the kernels take.  Column panels in sets of
+// 8, row tiles in sets of 4, row-tile-fastest inside such a 4 x 8 block.  The 32 compute units of an XCD then work on
+// one block at a time and fetch 4 + 8 operand panels for 32 tiles; with many row tiles (the weight gradient: hidden /
+// 256 of them) plain row-tile-fastest order would have them on 16 x 2 tiles and fetch 18.  Up to 4 row tiles per group
+// the two orders are the same.  A single row tile left over after the blocks of 4 (a group of 5 or 9 row tiles:
+// typically the small tail tile of a ragged group) joins the last block instead of forming one of its own, so it runs
+// beside the tiles whose column panels it shares (measured: 0.2 to 0.4 % per layer step).
+__host__ __device__ __forceinline__ void tile_order(int r, int R, int C, int &row_tile, int &col_tile) {
+    constexpr int BR = 4, BC = 8;      // measured against 8 x 4, 8 x 8, 2 x 16 and 4 x 16: the fastest for all three products
+    const int cg = r / (BC * R);
+    const int rem = r - cg * BC * R;
+    const int wc = C - BC * cg < BC ? C - BC * cg : BC;    // column panels in this set
+    int nb = (R + BR - 1) / BR;
+    if (R > BR && R % BR == 1) nb -= 1;                     // a single left-over row tile joins the block before it
+    int rb = rem / (BR * wc);
+    rb = rb > nb - 1 ? nb - 1 : rb;
+    const int rem2 = rem - rb * BR * wc;
+    const int hr = rb == nb - 1 ? R - BR * rb : BR;        // row tiles in this block
+    const int lc = rem2 / hr;
+    col_tile = BC * cg + lc;
+    row_tile = BR * rb + (rem2 - lc * hr);
+}
+
 // Map this workgroup to its tile.  Workgroup b runs on XCD b % 8 (round-robin dispatch) and takes slot
 // b / 8 of that XCD's slot sequence.  Every XCD walks the groups in the same order and owns one contiguous
 // eighth of each group's tiles (in the blocked order below), so concurrently running
@@ -108,29 +131,7 @@ __device__ __forceinline__ TileCoord locate_tile(const TileTable *table) {
     tc.e = table->entries[lo];
     const int r = xcd * tc.e.share + (slot - tc.e.tile_begin);
     if (r >= tc.e.num_tiles) return tc;
-    // Tile order inside a group: column panels in sets of 8, row tiles in sets of 4, row-tile-fastest inside such a
-    // 4 x 8 block.  The 32 compute units of an XCD then work on one block at a time and fetch 4 + 8 operand panels
-    // for 32 tiles; with many row tiles (the weight gradient: hidden / 256 of them) plain row-tile-fastest order
-    // would have them on 16 x 2 tiles and fetch 18.  Up to 4 row tiles per group the two orders are the same.  A single
-    // row tile left over after the blocks of 4 (a group of 5 or 9 row tiles: typically the small tail tile of a ragged
-    // group) joins the last block instead of forming one of its own, so it runs beside the tiles whose column panels
-    // it shares (measured: 0.2 to 0.4 % per layer step).
-    {
-        constexpr int BR = 4, BC = 8;      // measured against 8 x 4, 8 x 8, 2 x 16 and 4 x 16: the fastest for all three products
-        const int R = tc.e.num_row_tiles, C = tc.e.num_tiles / R;
-        const int cg = r / (BC * R);
-        const int rem = r - cg * BC * R;
-        const int wc = C - BC * cg < BC ? C - BC * cg : BC;    // column panels in this set
-        int nb = (R + BR - 1) / BR;
-        if (R > BR && R % BR == 1) nb -= 1;                     // a single left-over row tile joins the block before it
-        int rb = rem / (BR * wc);
-        rb = rb > nb - 1 ? nb - 1 : rb;
-        const int rem2 = rem - rb * BR * wc;
-        const int hr = rb == nb - 1 ? R - BR * rb : BR;        // row tiles in this block
-        const int lc = rem2 / hr;
-        tc.col_tile = BC * cg + lc;
-        tc.row_tile = BR * rb + (rem2 - lc * hr);
-    }
+    tile_order(r, tc.e.num_row_tiles, tc.e.num_tiles / tc.e.num_row_tiles, tc.row_tile, tc.col_tile);
     tc.tile_rows = (tc.e.tail_rows != 0 && tc.row_tile == tc.e.num_row_tiles - 1) ? tc.e.tail_rows : tc.e.tile_rows;
     tc.valid = true;
     return tc;

@@ -70,3 +70,28 @@ def test_workspace_size_and_validation_are_host_only():
     assert rc != 0 and b"topk" in lib.ms_last_error()
     with pytest.raises(_lib.MindSpeedAmdError):
         _lib.check(rc, "ms_moe_token_unpermute")
+
+
+def test_tile_order_visits_every_tile_once():
+    """The order in which the grouped-matmul kernels walk the tiles of a group (blocks of 4 row tiles x 8 column
+    panels, partly filled blocks at both edges, a single left-over row tile joining the last block) is a bijection
+    for every group shape up to 40 x 40, and where the sides are multiples of 4 and 8 every run of 32 consecutive
+    indices is one 4 x 8 block."""
+    lib = _lib.load()
+    row, col = ctypes.c_int(-1), ctypes.c_int(-1)
+    for R in range(1, 41):
+        for C in range(1, 41):
+            seen = set()
+            order = []
+            for i in range(R * C):
+                assert lib.ms_gmm_tile_order(R, C, i, ctypes.byref(row), ctypes.byref(col)) == 0
+                assert 0 <= row.value < R and 0 <= col.value < C, (R, C, i, row.value, col.value)
+                seen.add((row.value, col.value))
+                order.append((row.value, col.value))
+            assert len(seen) == R * C, (R, C)
+            if R % 4 == 0 and C % 8 == 0:
+                for b in range(0, R * C, 32):
+                    chunk = order[b:b + 32]
+                    assert len({r for r, _ in chunk}) == 4 and len({c for _, c in chunk}) == 8, (R, C, b)
+    assert lib.ms_gmm_tile_order(4, 4, 16, ctypes.byref(row), ctypes.byref(col)) != 0
+    assert lib.ms_gmm_tile_order(0, 4, 0, ctypes.byref(row), ctypes.byref(col)) != 0
