@@ -13,8 +13,10 @@
 //     by gmm_split_reduce_kernel) so that they fill one round instead of
 //     running long on a few compute units.
 //   * every XCD takes a contiguous eighth of every group's tiles (workgroup b
-//     runs on XCD b % 8), row-tile-fastest inside a column panel, so the
-//     workgroups running together on an XCD share operand panels in its L2.
+//     runs on XCD b % 8), in blocks of 4 row tiles x 8 column panels, so the
+//     workgroups running together on an XCD share operand panels in its L2;
+//     with many small groups whole groups are dealt out to single XCDs instead
+//     (one list of entries per XCD).
 //   * the fast 16-bit kernels live in gmm_fast.hip.  Here: gmm16_kernel, the
 //     16-bit kernel for operands that do not allow 16-byte vector access
 //     (element-wise guarded loads, operands that are not contiguous along the
@@ -112,7 +114,8 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
                                                            int split_tails, int tails_last_below,
                                                            int64_t b_stride_group, int64_t c_stride_group,
                                                            const int64_t *__restrict__ b_offsets, TileTable *table,
-                                                           SplitTail *split_records, int split_cols, int split_cus) {
+                                                           SplitTail *split_records, int split_cols, int split_cus,
+                                                           GroupEntry *members) {
     extern __shared__ int64_t ends[];          // [num_groups] clamped end offset of every group
     __shared__ int64_t scratch64[4];
     __shared__ ScanItem scratch_item[4];
@@ -197,6 +200,85 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
     const int part_len = split_parts > 1 ? (steps + split_parts - 1) / split_parts * BK : k;
     const int used_parts = split_parts > 1 ? (k + part_len - 1) / part_len : 1;
 
+    // ---- whole groups to single XCDs ----------------------------------------------------------------
+    // With many groups an XCD's eighth of a group is only a handful of tiles, and every XCD fetches nearly all of the
+    // group's operand panels into its own L2.  Split on rows only (there a group's tiles are its work): the groups are
+    // ranked by their tile counts and dealt out by rank; every XCD gets a list of its own and takes all tiles of its
+    // groups, so a group's operands are fetched by one XCD only.  Taken when no XCD ends up more than 3 % over the
+    // average (the launch's grid allows for 4 %); otherwise every group is cut in eight as usual.
+    __shared__ int keys[kMaxListGroups];
+    __shared__ int by_rank[kMaxListGroups];
+    __shared__ int rank_of[kMaxListGroups];
+    __shared__ int asg_xcd[kMaxListGroups];
+    __shared__ int asg_pos[kMaxListGroups];
+    __shared__ int asg_begin[kMaxListGroups];
+    __shared__ int xcd_load[8];
+    __shared__ int xcd_count[8];
+    __shared__ int lists_ok;
+    bool lists = false;
+    __shared__ int most_row_tiles;
+    if (tid == 0) most_row_tiles = 0;
+    __syncthreads();
+    if (members != nullptr && group_type == 0 && num_groups >= 16 && num_groups <= kMaxListGroups && !tails_last) {
+        int most = 0;
+        for (int g = g0; g < g1; ++g) {
+            const int rt = plan_of(g).row_tiles;
+            keys[g] = rt * num_col_tiles;
+            most = rt > most ? rt : most;
+        }
+        if (most > 0) atomicMax(&most_row_tiles, most);
+        __syncthreads();
+    }
+    // Only where it pays: a group of more than 8 row tiles has eighths of distinct row tiles anyway (every XCD then
+    // fetches its own rows of the group and only the weight panels eight times), and measured on a skewed workload
+    // whose tiles lie mostly in such groups the lists gain nothing.
+    if (members != nullptr && group_type == 0 && num_groups >= 16 && num_groups <= kMaxListGroups && !tails_last &&
+        most_row_tiles <= 8) {
+        for (int g = g0; g < g1; ++g) {
+            const int key = keys[g];
+            int rank = 0;
+#pragma unroll 8
+            for (int h = 0; h < num_groups; ++h) rank += (keys[h] > key || (keys[h] == key && h < g)) ? 1 : 0;
+            by_rank[rank] = g;
+            rank_of[g] = rank;
+        }
+        __syncthreads();
+        // Dealt out by rank, eight at a time, alternately ascending and descending over the XCDs (rank 0..7 to XCD
+        // 0..7, rank 8..15 to XCD 7..0, ...): every group finds its XCD, its place in that XCD's list and the tiles in
+        // front of it by itself.  Empty groups are ranked last and get no entry.
+        if (tid < 8) {
+            xcd_load[tid] = 0;
+            xcd_count[tid] = 0;
+        }
+        __syncthreads();
+        for (int g = g0; g < g1; ++g) {
+            const int rank = rank_of[g];
+            const int round = rank >> 3;
+            const int x = (round & 1) ? 7 - (rank & 7) : (rank & 7);
+            int begin = 0;
+            for (int o = 0; o < round; ++o) begin += keys[by_rank[o * 8 + ((o & 1) ? 7 - x : x)]];
+            asg_xcd[g] = keys[g] != 0 ? x : -1;
+            asg_pos[g] = round;
+            asg_begin[g] = begin;
+            if (keys[g] != 0) {
+                atomicAdd(&xcd_load[x], keys[g]);
+                atomicAdd(&xcd_count[x], 1);
+            }
+        }
+        __syncthreads();
+        if (tid == 0) {
+            long long total = 0;
+            int max_load = 0;
+            for (int q = 0; q < 8; ++q) {
+                total += xcd_load[q];
+                max_load = xcd_load[q] > max_load ? xcd_load[q] : max_load;
+            }
+            lists_ok = total > 0 && static_cast<long long>(max_load) * 800 <= total * 103 ? 1 : 0;
+        }
+        __syncthreads();
+        lists = lists_ok != 0;
+    }
+
     // What every group emits in each pass.
     auto item_of = [&](const GroupPlan &p) {
         ScanItem it{};
@@ -230,6 +312,64 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
         if (idx < max_entries) table->entries[idx] = e;
         if (idx < 16) table->begins[idx] = e.tile_begin;
     };
+    if (lists) {
+        const int stride = num_groups + 1;      // a list may hold nearly every group, and the zero-fill pseudo-group
+        for (int g = g0; g < g1; ++g) {
+            if (asg_xcd[g] < 0) continue;
+            const GroupPlan p = plan_of(g);
+            const int prev = g > 0 ? static_cast<int>(ends[g - 1]) : 0;
+            GroupEntry f{};
+            f.tile_rows = tile_rows;
+            f.row_begin = prev;
+            f.row_end = static_cast<int>(ends[g]);
+            f.red_begin = 0;
+            f.red_end = k;
+            f.b_off = b_offsets != nullptr ? b_offsets[g] : g * b_stride_group;
+            f.num_row_tiles = p.row_tiles;
+            f.tail_rows = p.tail_rows;
+            f.num_tiles = p.row_tiles * num_col_tiles;
+            f.share = f.num_tiles;
+            f.whole = 1;
+            f.tile_begin = asg_begin[g];
+            members[static_cast<int64_t>(asg_xcd[g]) * stride + asg_pos[g]] = f;
+        }
+        if (tid == 0) {
+            int slots = 0;
+            for (int q = 0; q < 8; ++q) slots = xcd_load[q] > slots ? xcd_load[q] : slots;
+            int counts[8];
+            for (int q = 0; q < 8; ++q) counts[q] = xcd_count[q];
+            const int last_end = static_cast<int>(ends[num_groups - 1]);
+            if (last_end < m) {                 // rows past the last offset: zero-fill, an eighth for every XCD behind its groups
+                GroupEntry e{};
+                e.row_begin = last_end;
+                e.row_end = m;
+                e.tile_rows = tile_rows;
+                const int len = m - last_end;
+                e.num_row_tiles = (len + tile_rows - 1) / tile_rows;
+                const int rem = len - (e.num_row_tiles - 1) * tile_rows;
+                e.tail_rows = !split_tails ? 0 : (rem <= 64 ? 64 : (rem <= 128 ? 128 : 0));
+                e.num_tiles = e.num_row_tiles * num_col_tiles;
+                e.share = (e.num_tiles + 7) >> 3;
+                int most = 0;
+                for (int q = 0; q < 8; ++q) {
+                    e.tile_begin = xcd_load[q];
+                    members[static_cast<int64_t>(q) * stride + counts[q]] = e;
+                    counts[q] += 1;
+                    most = xcd_load[q] + e.share > most ? xcd_load[q] + e.share : most;
+                }
+                slots = most;
+            }
+            table->slots_per_xcd = slots;
+            table->num_entries = 0;
+            table->num_split_tails = 0;
+            table->lists_off = static_cast<int>(reinterpret_cast<char *>(members) - reinterpret_cast<char *>(table));
+            table->list_stride = stride;
+            for (int q = 0; q < 8; ++q) table->list_count[q] = counts[q];
+            for (int i = 0; i < 8; ++i) table->zeros[i] = 0;
+            for (int i = 0; i < 16; ++i) table->begins[i] = 0x7fffffff;
+        }
+        return;
+    } else
     for (int g = g0; g < g1; ++g) {
         const GroupPlan p = plan_of(g);
         const ScanItem it = item_of(p);
@@ -308,6 +448,8 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
         table->slots_per_xcd = slots;
         table->num_entries = n;
         table->num_split_tails = all.tails;
+        table->lists_off = 0;
+        table->list_stride = 0;
         for (int i = 0; i < 8; ++i) table->zeros[i] = 0;
         for (int i = n; i < 16; ++i) table->begins[i] = 0x7fffffff;
     }
@@ -393,7 +535,7 @@ struct TileLoader {
 template <int DT, bool A_RED, bool B_RED, int OUT>
 __global__ __launch_bounds__(256) void gmm16_kernel(const GmmArgs p) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
-    const TileCoord tc = locate_tile(p.table);
+    const TileCoord tc = locate_tile<false>(p.table);
     if (!tc.valid) return;
 
     const int tid = threadIdx.x;
@@ -527,7 +669,7 @@ template <bool ACC>
 __global__ __launch_bounds__(256) void gmm32_kernel(const GmmArgs p) {
     __shared__ float sa[FK][FPITCH];
     __shared__ float sb[FK][FPITCH];
-    const TileCoord tc = locate_tile(p.table);
+    const TileCoord tc = locate_tile<false>(p.table);
     if (!tc.valid) return;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -633,8 +775,13 @@ constexpr size_t table_bytes(int64_t num_groups) {
 // records of the split tails
 constexpr size_t offsets_pos(int64_t num_groups) { return (table_bytes(num_groups) + 7) & ~static_cast<size_t>(7); }
 constexpr size_t split_records_pos(int64_t num_groups) { return offsets_pos(num_groups) + kMaxWeightList * sizeof(int64_t); }
-constexpr size_t workspace_need(int64_t num_groups) {
+constexpr size_t members_pos(int64_t num_groups) {
     return split_records_pos(num_groups) + static_cast<size_t>(num_groups) * sizeof(SplitTail);
+}
+// ... then the eight per-XCD lists of entries (whole groups dealt out to single XCDs): num_groups + 1 entries each
+constexpr size_t workspace_need(int64_t num_groups) {
+    return members_pos(num_groups) +
+           (num_groups >= 16 && num_groups <= kMaxListGroups ? static_cast<size_t>(8 * (num_groups + 1)) * sizeof(GroupEntry) : 0);
 }
 // ... and, for launches that may split the reduction of their small tail tiles, the fp32 partial sums behind that
 constexpr size_t split_ws_pos(int64_t num_groups) { return (workspace_need(num_groups) + 255) & ~static_cast<size_t>(255); }
@@ -852,12 +999,16 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
         split_records = reinterpret_cast<SplitTail *>(static_cast<char *>(workspace) + split_records_pos(num_groups));
         split_ws = reinterpret_cast<float *>(static_cast<char *>(workspace) + split_ws_pos(num_groups));
     }
+    // whole groups to single XCDs (fast kernels only): room for the lists lies in every workspace of 16 to 512 groups
+    GroupEntry *members = num_groups >= 16 && num_groups <= kMaxListGroups
+        ? reinterpret_cast<GroupEntry *>(static_cast<char *>(workspace) + members_pos(num_groups)) : nullptr;
     auto schedule = [&](int split_tails) -> int {
         hipLaunchKernelGGL(gmm_schedule_kernel, dim3(1), dim3(256), static_cast<size_t>(num_groups) * sizeof(int64_t),
                            stream, group_list, group_list_type, group_type, static_cast<int>(num_groups),
                            static_cast<int>(m), static_cast<int>(k), tile_rows, static_cast<int>(num_col_tiles),
                            split_tails, kTailsLastRounds * num_cus, w_stride_group, c_stride_group, b_offsets, table,
-                           split_tails ? split_records : nullptr, static_cast<int>(n), num_cus);
+                           split_tails ? split_records : nullptr, static_cast<int>(n), num_cus,
+                           split_tails ? members : nullptr);
         MS_CHECK_LAUNCH("gmm_schedule_kernel");
         return MS_OK;
     };
@@ -876,9 +1027,11 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     args.num_col_tiles = static_cast<int>(num_col_tiles);
     // slots per XCD: every entry rounds its tiles up to a multiple of 8; a launch that may split its tail tiles has up
     // to kMaxSplit entries per tail and up to kSplitCus more tiles
+    // (a launch that may deal whole groups out to the XCDs has up to 1.03 times an eighth of all tiles as slots)
+    const int64_t slot_tiles = members != nullptr ? tiles_bound + tiles_bound / 25 : tiles_bound;
     const unsigned grid = split_ws == nullptr
-        ? static_cast<unsigned>((ceil_div(tiles_bound, 8) + 2 * num_groups + 2) * 8)
-        : static_cast<unsigned>((ceil_div(tiles_bound + kSplitCus, 8) + (1 + kMaxSplit) * num_groups + 2) * 8);
+        ? static_cast<unsigned>((ceil_div(slot_tiles, 8) + 2 * num_groups + 2) * 8)
+        : static_cast<unsigned>((ceil_div(slot_tiles + kSplitCus, 8) + (1 + kMaxSplit) * num_groups + 2) * 8);
 
     if (swiglu != nullptr) {
         args.cols = static_cast<int>(n / 2);
@@ -1005,7 +1158,10 @@ extern "C" int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int6
 // GPU.  In host code the array's name is only a handle for hipGetSymbolAddress; kernels get the address that call
 // returned, looked up once per device.
 constexpr int kNoAllocMaxGroups = 1024;
-constexpr size_t kScratchBytes = (workspace_need(kNoAllocMaxGroups) + 255) & ~static_cast<size_t>(255);
+// (the need is largest either for the most groups or for the most groups that may get per-XCD lists)
+constexpr size_t kScratchNeed = workspace_need(kNoAllocMaxGroups) > workspace_need(kMaxListGroups)
+    ? workspace_need(kNoAllocMaxGroups) : workspace_need(kMaxListGroups);
+constexpr size_t kScratchBytes = (kScratchNeed + 255) & ~static_cast<size_t>(255);
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 namespace {

@@ -23,7 +23,7 @@ struct GroupEntry {
     int share;               // ceil(num_tiles / 8): tiles of this group handled by each XCD
     int split;               // 0, or 1 + the part number of a small tail tile whose reduction is split: such a
                              // tile writes fp32 partial sums to the split workspace (c_off then points there)
-    int reserved;
+    int whole;               // entry of an XCD's own list: 1 = that XCD takes all tiles of the group, 0 = its eighth
     int64_t b_off;           // element offset of the group's weight block
     int64_t c_off;           // element offset of the group's output block
 };
@@ -38,14 +38,20 @@ constexpr int kSplitRows = 128;          // rows reserved per (tail, part) pair:
 constexpr int kMaxSplit = 4;             // most parts a reduction is split into
 constexpr int kSplitCus = 256;           // a launch's split parts never number more than this (one round of MI355X's CUs)
 constexpr int kSplitMinRed = 2048;       // shortest reduction range worth a part of its own
+constexpr int kMaxListGroups = 256;      // most groups that may be dealt out whole to single XCDs (ranked by counting,
+                                         // dealt out by one thread)
 
 struct TileTable {
     int slots_per_xcd;       // sum of the entries' shares
     int num_entries;
     int num_split_tails;     // tail tile rows whose reduction was split (entries of the SplitTail array in use)
-    int pad[5];
+    int lists_off;           // 0, or the byte offset from the table to eight lists of entries, one per XCD (whole groups
+                             // dealt out to single XCDs); `entries` is then unused
+    int list_stride;         // entries reserved per list
+    int pad[3];
     int zeros[8];            // always zero: source of out-of-range operand chunks (holds an aligned 16-byte block)
     int begins[16];          // tile_begin of the first 16 entries (INT_MAX past the last): one load finds the entry
+    int list_count[8];       // entries in use in every XCD's list
     GroupEntry entries[1];
 };
 
@@ -105,16 +111,38 @@ __host__ __device__ __forceinline__ void tile_order(int r, int R, int C, int &ro
 }
 
 // Map this workgroup to its tile.  Workgroup b runs on XCD b % 8 (round-robin dispatch) and takes slot
-// b / 8 of that XCD's slot sequence.  Every XCD walks the groups in the same order and owns one contiguous
-// eighth of each group's tiles (in the blocked order below), so concurrently running
+// b / 8 of that XCD's slot sequence.  Normally every XCD walks the groups in the same order and owns one contiguous
+// eighth of each group's tiles (in the blocked order above), so concurrently running
 // workgroups of an XCD share operand panels in that XCD's L2, and every XCD gets an equal part of every
-// group however unequal the groups are.
+// group however unequal the groups are.  With many groups the schedule may instead deal whole groups out to single
+// XCDs (every XCD then has a list of its own): a group's operands are fetched into one L2 instead of eight.
+// LISTS: the kernel may meet per-XCD lists (the fast kernels of the split on rows); the others are compiled without that
+// path, which costs the weight-gradient kernel 0.3 us per tile at its start when it is merely present.
+template <bool LISTS>
 __device__ __forceinline__ TileCoord locate_tile(const TileTable *table) {
     TileCoord tc;
     tc.valid = false;
     const int xcd = blockIdx.x & 7;
     const int slot = blockIdx.x >> 3;
     if (slot >= table->slots_per_xcd) return tc;
+    if (LISTS && table->num_entries == 0) {     // per-XCD lists (the common table is empty then); no further header
+                                                // field is read on the way to the common case
+        const GroupEntry *list = reinterpret_cast<const GroupEntry *>(reinterpret_cast<const char *>(table) + table->lists_off) +
+                                 static_cast<int64_t>(xcd) * table->list_stride;
+        int lo = 0, hi = table->list_count[xcd];
+        if (hi == 0) return tc;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (list[mid].tile_begin <= slot) lo = mid; else hi = mid;
+        }
+        tc.e = list[lo];
+        const int r = slot - tc.e.tile_begin + (tc.e.whole != 0 ? 0 : xcd * tc.e.share);
+        if (r >= tc.e.num_tiles || (tc.e.whole == 0 && slot - tc.e.tile_begin >= tc.e.share)) return tc;
+        tile_order(r, tc.e.num_row_tiles, tc.e.num_tiles / tc.e.num_row_tiles, tc.row_tile, tc.col_tile);
+        tc.tile_rows = (tc.e.tail_rows != 0 && tc.row_tile == tc.e.num_row_tiles - 1) ? tc.e.tail_rows : tc.e.tile_rows;
+        tc.valid = true;
+        return tc;
+    }
     // last entry with tile_begin <= slot.  Up to 16 entries (8 experts with their tail tiles) their begins lie in the
     // table's header and are fetched at once, instead of one dependent load per step of a binary search.
     int lo = 0;

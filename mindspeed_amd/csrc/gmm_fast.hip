@@ -751,7 +751,7 @@ template <int DT, bool A_RED, bool B_RED, int OUT>
 __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     MS_TRACE(1);
-    const TileCoord tc = locate_tile(p.table);
+    const TileCoord tc = locate_tile<A_RED>(p.table);   // A_RED: the split on rows, the only form with per-XCD lists
     if (!tc.valid) return;
     MS_TRACE(2);
     if (tc.tile_rows == 256) {

@@ -99,6 +99,9 @@ GMM_CASES = [
     # forward (4 + 5), 5 x 10 in the weight gradient (one block of 5), and a ragged pair of groups with 5 row tiles each
     (2300, 1280, 2560, 1, "equal"),
     (2100, 768, 1024, 2, "equal"),
+    # many groups of a few row tiles each: whole groups go to single XCDs (lists per XCD) in forward and dX
+    (32768, 256, 1280, 64, "equal"),
+    (20000, 320, 768, 24, "equal"),
 ]
 
 
@@ -343,3 +346,25 @@ def test_split_tail_tiles_with_rows_past_the_last_offset(device):
             full[end - rem:end] = False
     full[covered:] = False
     assert torch.equal(plain[full.to(device)], split[full.to(device)])
+
+
+def test_many_small_groups_take_whole_groups_per_xcd(device):
+    """Near-equal ragged groups of two to five row tiles, 40 of them, and rows past the last offset: the launch deals
+    whole groups out to single XCDs; forward, dX and dW against the oracle, the uncovered rows zero."""
+    say("many small groups")
+    gen = torch.Generator().manual_seed(21)
+    E, K, N, extra = 40, 384, 1536, 300
+    counts = torch.randint(600, 1200, (E,), generator=gen)
+    M = int(counts.sum())
+    x = torch.randn(M + extra, K, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(E, K, N, generator=gen) * 0.05).to(torch.bfloat16)
+    gy = torch.randn(M + extra, N, generator=gen).to(torch.bfloat16)
+    xd, wd = x.to(device).requires_grad_(True), w.to(device).requires_grad_(True)
+    y = ops.npu_gmm_v2(xd, wd, group_list=counts.to(device), group_type=0)
+    y.backward(gy.to(device))
+    ey = O.grouped_matmul(x[:M], counts.tolist(), w)
+    assert rel_l2(y[:M], ey) <= TOL[torch.bfloat16]
+    assert torch.equal(y[M:].cpu(), torch.zeros(extra, N, dtype=torch.bfloat16))
+    edx, edw = O.gmm_backward(gy[:M], x[:M], w, torch.cumsum(counts, 0).tolist())
+    assert rel_l2(xd.grad[:M], edx) <= TOL[torch.bfloat16] and rel_l2(wd.grad, edw) <= TOL[torch.bfloat16]
+    assert torch.equal(xd.grad[M:].cpu(), torch.zeros(extra, K, dtype=torch.bfloat16))
