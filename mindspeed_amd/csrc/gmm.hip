@@ -219,21 +219,28 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
     __shared__ int most_row_tiles;
     if (tid == 0) most_row_tiles = 0;
     __syncthreads();
-    if (members != nullptr && group_type == 0 && num_groups >= 16 && num_groups <= kMaxListGroups && !tails_last) {
+    const bool lists_wanted = members != nullptr && num_groups >= 16 && num_groups <= kMaxListGroups && !tails_last;
+    const int out_tiles = ((k + tile_rows - 1) / tile_rows) * num_col_tiles;     // split on the reduction dim: tiles per group
+    if (lists_wanted) {
         int most = 0;
         for (int g = g0; g < g1; ++g) {
-            const int rt = plan_of(g).row_tiles;
-            keys[g] = rt * num_col_tiles;
-            most = rt > most ? rt : most;
+            if (group_type == 0) {
+                const int rt = plan_of(g).row_tiles;
+                keys[g] = rt * num_col_tiles;
+                most = rt > most ? rt : most;
+            } else {
+                const int prev = g > 0 ? static_cast<int>(ends[g - 1]) : 0;
+                keys[g] = static_cast<int>(ends[g]) - prev;              // the work of a group's tiles: its reduction length
+            }
         }
         if (most > 0) atomicMax(&most_row_tiles, most);
         __syncthreads();
     }
-    // Only where it pays: a group of more than 8 row tiles has eighths of distinct row tiles anyway (every XCD then
-    // fetches its own rows of the group and only the weight panels eight times), and measured on a skewed workload
-    // whose tiles lie mostly in such groups the lists gain nothing.
-    if (members != nullptr && group_type == 0 && num_groups >= 16 && num_groups <= kMaxListGroups && !tails_last &&
-        most_row_tiles <= 8) {
+    // Only where it pays.  Split on rows: a group of more than 8 row tiles has eighths of distinct row tiles anyway
+    // (every XCD then fetches its own rows of the group and only the weight panels eight times), and measured on a
+    // skewed workload whose tiles lie mostly in such groups the lists gain nothing.  Split on the reduction dim: an
+    // output block of at most 256 tiles (an eighth of it is then at most one block of 4 x 8).
+    if (lists_wanted && (group_type == 0 ? most_row_tiles <= 8 : out_tiles <= 256)) {
         for (int g = g0; g < g1; ++g) {
             const int key = keys[g];
             int rank = 0;
@@ -255,12 +262,16 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
             const int rank = rank_of[g];
             const int round = rank >> 3;
             const int x = (round & 1) ? 7 - (rank & 7) : (rank & 7);
-            int begin = 0;
-            for (int o = 0; o < round; ++o) begin += keys[by_rank[o * 8 + ((o & 1) ? 7 - x : x)]];
-            asg_xcd[g] = keys[g] != 0 ? x : -1;
+            int begin = round * out_tiles;        // split on the reduction dim: every group has the same tiles
+            if (group_type == 0) {
+                begin = 0;
+                for (int o = 0; o < round; ++o) begin += keys[by_rank[o * 8 + ((o & 1) ? 7 - x : x)]];
+            }
+            const bool has_entry = group_type == 2 || keys[g] != 0;   // (an empty group's output block is written as zeros)
+            asg_xcd[g] = has_entry ? x : -1;
             asg_pos[g] = round;
             asg_begin[g] = begin;
-            if (keys[g] != 0) {
+            if (has_entry) {
                 atomicAdd(&xcd_load[x], keys[g]);
                 atomicAdd(&xcd_count[x], 1);
             }
@@ -320,11 +331,19 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
             const int prev = g > 0 ? static_cast<int>(ends[g - 1]) : 0;
             GroupEntry f{};
             f.tile_rows = tile_rows;
-            f.row_begin = prev;
-            f.row_end = static_cast<int>(ends[g]);
-            f.red_begin = 0;
-            f.red_end = k;
-            f.b_off = b_offsets != nullptr ? b_offsets[g] : g * b_stride_group;
+            if (group_type == 0) {
+                f.row_begin = prev;
+                f.row_end = static_cast<int>(ends[g]);
+                f.red_begin = 0;
+                f.red_end = k;
+                f.b_off = b_offsets != nullptr ? b_offsets[g] : g * b_stride_group;
+            } else {
+                f.row_begin = 0;
+                f.row_end = k;
+                f.red_begin = prev;
+                f.red_end = static_cast<int>(ends[g]);
+                f.c_off = g * c_stride_group;
+            }
             f.num_row_tiles = p.row_tiles;
             f.tail_rows = p.tail_rows;
             f.num_tiles = p.row_tiles * num_col_tiles;
@@ -335,11 +354,14 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
         }
         if (tid == 0) {
             int slots = 0;
-            for (int q = 0; q < 8; ++q) slots = xcd_load[q] > slots ? xcd_load[q] : slots;
+            for (int q = 0; q < 8; ++q) {
+                const int tiles_q = group_type == 0 ? xcd_load[q] : xcd_count[q] * out_tiles;
+                slots = tiles_q > slots ? tiles_q : slots;
+            }
             int counts[8];
             for (int q = 0; q < 8; ++q) counts[q] = xcd_count[q];
             const int last_end = static_cast<int>(ends[num_groups - 1]);
-            if (last_end < m) {                 // rows past the last offset: zero-fill, an eighth for every XCD behind its groups
+            if (group_type == 0 && last_end < m) {                 // rows past the last offset: zero-fill, an eighth for every XCD behind its groups
                 GroupEntry e{};
                 e.row_begin = last_end;
                 e.row_end = m;
@@ -1000,7 +1022,10 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
         split_ws = reinterpret_cast<float *>(static_cast<char *>(workspace) + split_ws_pos(num_groups));
     }
     // whole groups to single XCDs (fast kernels only): room for the lists lies in every workspace of 16 to 512 groups
-    GroupEntry *members = num_groups >= 16 && num_groups <= kMaxListGroups
+    // (the split on the reduction dim has a kernel variant with that lookup only for the layout of the weight gradient,
+    // both operands contiguous along their outer dims)
+    GroupEntry *members = num_groups >= 16 && num_groups <= kMaxListGroups &&
+                                  (group_type == 0 || (a_stride_row == 1 && b_stride_col == 1 && a_stride_red != 1 && b_stride_red != 1))
         ? reinterpret_cast<GroupEntry *>(static_cast<char *>(workspace) + members_pos(num_groups)) : nullptr;
     auto schedule = [&](int split_tails) -> int {
         hipLaunchKernelGGL(gmm_schedule_kernel, dim3(1), dim3(256), static_cast<size_t>(num_groups) * sizeof(int64_t),
@@ -1118,7 +1143,7 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     if (int rc = schedule(fast ? 1 : 0)) return rc;
     if (fast) {
         args.split_ws = split_ws;
-        if (int rc = launch_gmm16_fast(stream, args, dtype, out, a_is_red, b_is_red, grid)) return rc;
+        if (int rc = launch_gmm16_fast(stream, args, dtype, out, a_is_red, b_is_red, grid, members != nullptr)) return rc;
         if (split_ws != nullptr) {
             // at most kSplitCus / (2 parts x column tiles) tails are ever split in one launch
             const int64_t max_tails = kSplitCus / (2 * num_col_tiles) < num_groups ? kSplitCus / (2 * num_col_tiles) : num_groups;

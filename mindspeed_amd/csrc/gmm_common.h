@@ -188,7 +188,9 @@ __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1
 
 // Fast 16-bit kernels (gmm_fast.hip).  Returns MS_OK after launching, or -1 if
 // this problem does not meet the fast kernels' alignment conditions.
+// lists: the table may come as per-XCD lists (only asked of the weight-gradient product, whose common kernel is compiled
+// without that lookup; the kernels of the split on rows always have it).
 int launch_gmm16_fast(hipStream_t stream, const GmmArgs &args, int dtype, int out_mode, bool a_red, bool b_red,
-                      unsigned grid);
+                      unsigned grid, bool lists = false);
 
 }  // namespace ms

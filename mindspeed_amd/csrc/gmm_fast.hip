@@ -747,11 +747,13 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
     }
 }
 
-template <int DT, bool A_RED, bool B_RED, int OUT>
+// LISTS: the launch may come with per-XCD lists of entries.  Always so for the split on rows (A_RED); the weight-gradient
+// product has a variant of its own for launches of many groups, so that the common one does not carry that lookup.
+template <int DT, bool A_RED, bool B_RED, int OUT, bool LISTS = A_RED>
 __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     MS_TRACE(1);
-    const TileCoord tc = locate_tile<A_RED>(p.table);   // A_RED: the split on rows, the only form with per-XCD lists
+    const TileCoord tc = locate_tile<LISTS>(p.table);
     if (!tc.valid) return;
     MS_TRACE(2);
     if (tc.tile_rows == 256) {
@@ -783,7 +785,7 @@ __global__ __launch_bounds__(256) void gmm16_fast_kernel(const GmmArgs p) {
 }
 
 template <int DT, int OUT>
-int launch_fast(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red, unsigned grid) {
+int launch_fast(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red, unsigned grid, bool lists) {
     const void *fn;
     if constexpr (OUT == OUT_SWIGLU) {
         MS_REQUIRE(a_red && !b_red, MS_ERR_UNSUPPORTED, "ms_gmm_swiglu: operand layout not supported");
@@ -794,6 +796,7 @@ int launch_fast(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red,
     } else if (a_red && b_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, true, OUT>);
     else if (a_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, true, false, OUT>);
     else if (b_red) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, true, OUT>);
+    else if (lists) fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, false, OUT, true>);
     else fn = reinterpret_cast<const void *>(&gmm16_fast_kernel<DT, false, false, OUT>);
     int lds_bytes = 2 * ((a_red ? kRedTileBytes : kOuterTileBytes) + (b_red ? kRedTileBytes : kOuterTileBytes));
     if ((OUT == OUT_SAME || OUT == OUT_SWIGLU || OUT == OUT_SWIGLU_GRAD) && lds_bytes < kStageBytes) lds_bytes = kStageBytes;
@@ -810,23 +813,23 @@ int launch_fast(hipStream_t stream, const GmmArgs &args, bool a_red, bool b_red,
 }  // namespace
 
 int launch_gmm16_fast(hipStream_t stream, const GmmArgs &args, int dtype, int out_mode, bool a_red, bool b_red,
-                      unsigned grid) {
+                      unsigned grid, bool lists) {
     if (out_mode == OUT_SWIGLU) {
-        if (dtype == MS_BF16) return launch_fast<MS_BF16, OUT_SWIGLU>(stream, args, a_red, b_red, grid);
-        return launch_fast<MS_FP16, OUT_SWIGLU>(stream, args, a_red, b_red, grid);
+        if (dtype == MS_BF16) return launch_fast<MS_BF16, OUT_SWIGLU>(stream, args, a_red, b_red, grid, lists);
+        return launch_fast<MS_FP16, OUT_SWIGLU>(stream, args, a_red, b_red, grid, lists);
     }
     if (out_mode == OUT_SWIGLU_GRAD) {
-        if (dtype == MS_BF16) return launch_fast<MS_BF16, OUT_SWIGLU_GRAD>(stream, args, a_red, b_red, grid);
-        return launch_fast<MS_FP16, OUT_SWIGLU_GRAD>(stream, args, a_red, b_red, grid);
+        if (dtype == MS_BF16) return launch_fast<MS_BF16, OUT_SWIGLU_GRAD>(stream, args, a_red, b_red, grid, lists);
+        return launch_fast<MS_FP16, OUT_SWIGLU_GRAD>(stream, args, a_red, b_red, grid, lists);
     }
     if (dtype == MS_BF16) {
-        if (out_mode == OUT_SAME) return launch_fast<MS_BF16, OUT_SAME>(stream, args, a_red, b_red, grid);
-        if (out_mode == OUT_F32) return launch_fast<MS_BF16, OUT_F32>(stream, args, a_red, b_red, grid);
-        return launch_fast<MS_BF16, ACC_F32>(stream, args, a_red, b_red, grid);
+        if (out_mode == OUT_SAME) return launch_fast<MS_BF16, OUT_SAME>(stream, args, a_red, b_red, grid, lists);
+        if (out_mode == OUT_F32) return launch_fast<MS_BF16, OUT_F32>(stream, args, a_red, b_red, grid, lists);
+        return launch_fast<MS_BF16, ACC_F32>(stream, args, a_red, b_red, grid, lists);
     }
-    if (out_mode == OUT_SAME) return launch_fast<MS_FP16, OUT_SAME>(stream, args, a_red, b_red, grid);
-    if (out_mode == OUT_F32) return launch_fast<MS_FP16, OUT_F32>(stream, args, a_red, b_red, grid);
-    return launch_fast<MS_FP16, ACC_F32>(stream, args, a_red, b_red, grid);
+    if (out_mode == OUT_SAME) return launch_fast<MS_FP16, OUT_SAME>(stream, args, a_red, b_red, grid, lists);
+    if (out_mode == OUT_F32) return launch_fast<MS_FP16, OUT_F32>(stream, args, a_red, b_red, grid, lists);
+    return launch_fast<MS_FP16, ACC_F32>(stream, args, a_red, b_red, grid, lists);
 }
 
 }  // namespace ms
