@@ -35,12 +35,12 @@ import sys
 import threading
 import time
 
-GEMM_KEYS = {  # template arguments <dtype, A reduction-contiguous, B reduction-contiguous, output mode>
-    "gmm16_fast_kernel<0, true, false, 0>": "gmm_fwd",
-    "gmm16_fast_kernel<0, true, true, 0>": "gmm_dx",
-    "gmm16_fast_kernel<0, false, false, 0>": "gmm_dw",
-    "gmm16_fast_kernel<0, true, false, 3>": "gmm_fwd_swiglu",
-    "gmm16_fast_kernel<0, true, true, 4>": "gmm_dx_swiglu",
+GEMM_KEYS = {  # first template arguments <dtype, A reduction-contiguous, B reduction-contiguous, output mode, ...>
+    "gmm16_fast_kernel<0, true, false, 0,": "gmm_fwd",
+    "gmm16_fast_kernel<0, true, true, 0,": "gmm_dx",
+    "gmm16_fast_kernel<0, false, false, 0,": "gmm_dw",
+    "gmm16_fast_kernel<0, true, false, 3,": "gmm_fwd_swiglu",
+    "gmm16_fast_kernel<0, true, true, 4,": "gmm_dx_swiglu",
 }
 
 

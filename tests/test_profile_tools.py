@@ -10,7 +10,7 @@ from mindspeed_amd import build, profile_tools
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = "Dispatch_Id,Kernel_Name,Counter_Name,Counter_Value\n"
-FWD = "void ms::(anonymous namespace)::gmm16_fast_kernel<0, true, false, 0>(ms::GmmArgs)"
+FWD = "void ms::(anonymous namespace)::gmm16_fast_kernel<0, true, false, 0, true>(ms::GmmArgs)"
 COPY = "ms::(anonymous namespace)::copy_bytes_kernel(char const*, char*, unsigned long)"
 
 
@@ -22,7 +22,7 @@ def _write(path, counter, rows):
 
 
 def test_short_name_strips_namespace_and_arguments():
-    assert profile_tools.short_name(FWD) == "gmm16_fast_kernel<0, true, false, 0>"
+    assert profile_tools.short_name(FWD) == "gmm16_fast_kernel<0, true, false, 0, true>"
 
 
 def test_traffic_scales_counters_by_the_copy_and_records_the_build(tmp_path):
