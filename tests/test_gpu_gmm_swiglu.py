@@ -24,6 +24,8 @@ CASES = [
     ([300, 212], 72, 136, torch.float16, torch.float32, 0),
     ([1024, 1000, 1048], 512, 1024, torch.bfloat16, torch.float32, 0),       # full tiles, many rounds
     ([40], 8, 8, torch.bfloat16, torch.float32, 0),                          # smallest legal sizes
+    # many small groups with enough tiles for several rounds: whole groups go to single XCDs (per-XCD lists)
+    ([520 + 13 * (i % 7) for i in range(32)], 256, 768, torch.bfloat16, torch.float32, 9),
 ]
 
 
@@ -110,6 +112,8 @@ MLP_CASES = [
     ([130, 256, 1, 300, 64, 0, 200, 73], 256, 384, torch.bfloat16, torch.bfloat16, 5),
     ([300, 212], 72, 136, torch.float16, torch.float32, 0),
     ([700, 1000, 348], 512, 1024, torch.bfloat16, torch.float32, 0),
+    # many small groups: per-XCD lists in the fused kernels, forward and backward
+    ([430 + 17 * (i % 5) for i in range(24)], 256, 512, torch.bfloat16, torch.float32, 6),
 ]
 
 

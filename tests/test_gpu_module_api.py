@@ -23,6 +23,7 @@ CASES = [
     ([130, 256, 1, 300, 64, 0, 200, 73], 256, 512, torch.bfloat16),   # fast path, ragged tails
     ([100, 28], 72, 136, torch.float16),
     ([40, 40, 40], 64, 64, torch.bfloat16),                    # K == N: orientation taken as [E, K, N]
+    ([430 + 17 * (i % 5) for i in range(24)], 256, 512, torch.bfloat16),   # many small groups: per-XCD lists
 ]
 
 
