@@ -183,19 +183,30 @@ def measure_routing_map_mode(cfg, device, x, idx, p, iters=20, warmup=5):
     }
 
 
-def run_layer(cfg, device, steps, warmup, fuse_activation=False, per_kernel=True):
+def run_layer(cfg, device, steps, warmup, fuse_activation=False, per_kernel=True, accumulate=None):
     """`warmup` untimed steps, exactly `steps` timed ones between two synchronisations, then (per_kernel) the same
     steps again with every op bracketed by two events on its launch stream.  Returns (ms per step, ms per step with
-    the event brackets or None, per-kernel table or None, the inputs)."""
+    the event brackets or None, per-kernel table or None, the inputs).
+    accumulate: None, or how the weight gradients reach fp32 `main_grad` buffers of the weights: "fused" = added by
+    the weight-gradient product itself (gemm_fusion), "separate" = 16-bit weight gradients and one torch add each."""
     from mindspeed_amd import flop_counter
     from mindspeed_amd.dispatcher import dispatch_mlp_combine
 
     x, p, idx, w1, w2, gy = make_inputs(cfg, device)
     leaves = [t.requires_grad_(True) for t in (x, p, w1, w2)]
+    if accumulate is not None:
+        for w in (w1, w2):
+            w.main_grad = torch.zeros(w.shape, dtype=torch.float32, device=device)
+            w.grad_added_to_main_grad = False
 
     def step():
-        out = dispatch_mlp_combine(leaves[0], idx, leaves[1], (leaves[2], leaves[3]), fuse_activation=fuse_activation)
-        return torch.autograd.grad(out, leaves, gy)
+        out = dispatch_mlp_combine(leaves[0], idx, leaves[1], (leaves[2], leaves[3]), fuse_activation=fuse_activation,
+                                   gemm_fusion=accumulate == "fused")
+        grads = torch.autograd.grad(out, leaves, gy)
+        if accumulate == "separate":
+            w1.main_grad.add_(grads[2])
+            w2.main_grad.add_(grads[3])
+        return grads
 
     for _ in range(warmup):
         step()
@@ -352,6 +363,16 @@ def main():
                                 "gemm_frac_of_mfma_peak": {k: ok[k]["frac_of_mfma_peak"]
                                                            for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok}}
                 torch.cuda.empty_cache()
+            # the same Mixtral step with the weight gradients accumulated into fp32 buffers (the reference's
+            # gradient-accumulation fusion, mindspeed/ops/gmm.py:56-89) by the product itself, against 16-bit
+            # weight gradients followed by one add each
+            acc = {}
+            for how in ("fused", "separate"):
+                ms, _, ok, _ = run_layer(cfg, device, steps=10, warmup=5, accumulate=how)
+                acc[how] = {"ms_per_step": round(ms, 4),
+                            "gmm_dw_tflops": ok["gmm_dw"]["tflops"] if "gmm_dw" in ok else None}
+                torch.cuda.empty_cache()
+            others["mixtral_fp32_grad_accumulation"] = acc
             result["other_workloads"] = others
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg)

@@ -1,10 +1,11 @@
 """Grouped-matmul launches of the Mixtral-shape expert MLP in isolation.
 
-    python -m mindspeed_amd.gmm_microbench [--mode fwd1|fwd2|dx1|dx2|dw1|dw2|library] [--data randn|small|ones|zeros]
+    python -m mindspeed_amd.gmm_microbench [--mode fwd1|fwd2|dx1|dx2|dw1|dw2|dw1acc|dw2acc|library] [--data randn|small|ones|zeros]
                                            [--counts 988,1074,...] [--iters 20] [--warmup 20]
 
 ``fwd1`` / ``dx1`` / ``dw1`` are the forward, dX and dW products of the first matmul
 (``[T, H] x [E, H, 2F]``), ``fwd2`` / ``dx2`` / ``dw2`` those of the second (``[T, F] x [E, F, H]``);
+``dw1acc`` / ``dw2acc`` are the weight gradients added in place to an fp32 buffer;
 ``library`` runs ``torch.bmm`` on the fc1-forward shape as E dense products, for orientation.
 ``--data`` sets the operand values only (the rate of the matrix cores on this board depends on them);
 ``--counts`` gives the rows per expert (default: equal shares).  Prints milliseconds per launch and TFLOP/s.
@@ -20,7 +21,7 @@ from .ops.gmm import gmm_raw
 
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--mode", default="fwd1", choices=["fwd1", "fwd2", "dx1", "dx2", "dw1", "dw2", "library"])
+    ap.add_argument("--mode", default="fwd1", choices=["fwd1", "fwd2", "dx1", "dx2", "dw1", "dw2", "dw1acc", "dw2acc", "library"])
     ap.add_argument("--data", default="randn", choices=["randn", "small", "ones", "zeros"])
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=20)
@@ -70,6 +71,12 @@ def main():
     elif a.mode == "dw2":
         x, dy = operand(T, F), operand(T, H)
         fn, flops = (lambda: gmm_raw(x.t(), dy, counts, 2, 1)), 2 * T * H * F
+    elif a.mode in ("dw1acc", "dw2acc"):
+        # the fp32 `+=` form of the weight gradient (npu_groupmatmul_add_fp32): the sums grow by one product per
+        # launch, which leaves fp32 range only after ~1e30 launches
+        x, dy = (operand(T, H), operand(T, 2 * F)) if a.mode == "dw1acc" else (operand(T, F), operand(T, H))
+        grad = torch.zeros(E, x.size(1), dy.size(1), device=dev, dtype=torch.float32)
+        fn, flops = (lambda: gmm_raw(x.t(), dy, counts, 2, 1, out=grad, accumulate=True)), 2 * T * x.size(1) * dy.size(1)
     else:
         x, w = operand(E, T // E, H), operand(E, H, 2 * F)
         fn, flops = (lambda: torch.bmm(x, w)), 2 * T * H * 2 * F

@@ -219,6 +219,48 @@ def test_gemm_fusion_accumulates_into_main_grad(device):
     assert rel_l2(param.main_grad, exp_main) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("K,N", [(600, 520), (256, 256), (1032, 392)])
+def test_groupmatmul_add_reduction_lengths(K, N, dtype, device):
+    """The fp32 `+=` form over groups of 0 to 1000 rows (none, one, three, four, five and many K steps: its first old
+    values are requested from inside the K loop only where a group has at least four), output blocks whose last row and
+    column tiles are partly filled, twice in a row into the same buffer."""
+    say("groupmatmul_add reduction lengths", K, N, dtype)
+    counts = [0, 1, 31, 32, 96, 127, 128, 129, 1000, 0, 160, 333]
+    M = sum(counts)
+    gen = torch.Generator().manual_seed(K + N)
+    x = torch.randn(M, K, generator=gen).to(dtype)
+    dy = torch.randn(M, N, generator=gen).to(dtype)
+    acc0 = torch.randn(len(counts) * K, N, generator=gen)
+    offsets = torch.cumsum(torch.tensor(counts), 0)
+    acc = acc0.clone().to(device)
+    xd, dyd, od = x.to(device), dy.to(device), offsets.to(device)
+    ops.npu_groupmatmul_add_fp32(xd, dyd, od, acc)
+    exp = O.groupmatmul_add_fp32(x, dy, offsets, acc0.clone())
+    assert rel_l2(acc, exp) <= 1e-5
+    empty = [g for g, c in enumerate(counts) if c == 0]
+    for g in empty:                                  # nothing added: the old values exactly
+        assert torch.equal(acc[g * K:(g + 1) * K].cpu(), acc0[g * K:(g + 1) * K])
+    ops.npu_groupmatmul_add_fp32(xd, dyd, od, acc)
+    exp2 = O.groupmatmul_add_fp32(x, dy, offsets, exp.clone())
+    assert rel_l2(acc, exp2) <= 1e-5
+
+
+def test_groupmatmul_add_many_groups(device):
+    """The fp32 `+=` form with 24 near-equal groups (whole output blocks dealt out to single XCDs)."""
+    say("groupmatmul_add many groups")
+    counts = [200 + 9 * (i % 7) for i in range(24)]
+    M, K, N = sum(counts), 512, 520
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    dy = torch.randn(M, N, generator=gen).to(torch.bfloat16)
+    acc0 = torch.randn(len(counts) * K, N, generator=gen)
+    offsets = torch.cumsum(torch.tensor(counts), 0)
+    acc = acc0.clone().to(device)
+    ops.npu_groupmatmul_add_fp32(x.to(device), dy.to(device), offsets.to(device), acc)
+    assert rel_l2(acc, O.groupmatmul_add_fp32(x, dy, offsets, acc0.clone())) <= 1e-5
+
+
 def test_linearity_at_mixtral_fc1_shape(device):
     """Full-size property check on the Mixtral fc1 shape: gmm(a*x1 + x2) == a*gmm(x1) + gmm(x2) within bf16
     rounding, and sampled rows against per-row fp32 matmuls."""
