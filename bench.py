@@ -63,6 +63,30 @@ def measured_traffic(workload, kernel):
     return data.get("bytes_per_launch", {}).get(workload, {}).get(kernel)
 
 
+def board_mfma_rate(seconds=2.0):
+    """What the matrix cores of this board reach by themselves on random bf16 operands: the stand-alone probe
+    `mindspeed_amd/probes/bin/mfma_power` (built by `__graft_entry__.build()`), a loop of v_mfma_f32_32x32x16_bf16
+    with no memory traffic on every CU, run for `seconds` as a child process.  The board's power limit holds the shader
+    clock below the 2.4 GHz that the published peak is quoted at, by an amount that depends on the operand values; this
+    is the rate that limit leaves to a kernel that does nothing but multiply.  None if the probe is not built."""
+    import re
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "mindspeed_amd", "probes", "bin", "mfma_power")
+    if not os.path.exists(exe):
+        return None
+    try:
+        res = subprocess.run([exe, "quick", str(seconds)], capture_output=True, text=True, timeout=60)
+    except (OSError, subprocess.TimeoutExpired):
+        return None
+    m = re.search(r"32x32x16 random: ([\d.]+) TFLOP/s\s+(-?[\d.]+) W\s+(-?[\d.]+) MHz", res.stdout)
+    if res.returncode != 0 or m is None:
+        return None
+    return {"tflops": float(m.group(1)), "board_watts": float(m.group(2)), "shader_mhz": float(m.group(3)),
+            "what": "v_mfma_f32_32x32x16_bf16 back to back on all CUs, random operands in registers, no memory "
+                    f"traffic, {seconds:g} s (mindspeed_amd/probes/mfma_power.hip)"}
+
+
 def _cpu_layer_once(cfg, sample, dtype=torch.float32):
     from oracle import moe_oracle as O
 
@@ -331,6 +355,10 @@ def main():
         torch.cuda.synchronize()
         result["copy_calibration_bytes"] = n
     if not args.no_extras:
+        probe = board_mfma_rate()
+        if probe is not None:
+            result["board_mfma_probe"] = probe
+            roofline["frac_of_board_mfma_probe"] = round(dom["tflops"] / probe["tflops"], 4)
         result["routing_map_mode"] = measure_routing_map_mode(cfg, device, x.detach(), idx, p.detach())
         # The permute / unpermute family by itself at this workload's shape: back-to-back launches through the C ABI
         # (the per-op figures under "kernels" are single launches inside the layer step, whose operands were last

@@ -3,6 +3,8 @@
 // Shows how far the matrix cores alone get before the board's power limit pulls the clock down, and that the limit
 // depends on the operand values.  Power and clock come from the amdgpu hwmon / sysfs files (read-only).
 // Build and run: python -m mindspeed_amd.probes run mfma_power
+// With arguments `quick SECONDS` only the 32x32x16 loop on random data runs, for that long (what a benchmark calls to
+// read the board it is running on).
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -66,11 +68,13 @@ static int read_sclk() {
 
 int main(int argc, char **argv) {
     glob_t g; if (glob("/sys/class/drm/card*/device/hwmon/hwmon*", 0, nullptr, &g) == 0 && g.gl_pathc) hwmon = g.gl_pathv[0];
+    const bool quick = argc >= 2 && strcmp(argv[1], "quick") == 0;
+    const double seconds = quick && argc >= 3 ? atof(argv[2]) : 4.0;
     const int n = 65536;
     std::vector<unsigned> h(n * 4);
     v16 *src; float *out;
     (void)hipMalloc(&src, n * 16); (void)hipMalloc(&out, 1 << 22);
-    for (int mode = 0; mode < 2; ++mode) {          // 0: random bf16 values ~N(0,1)-like bit patterns, 1: zeros
+    for (int mode = 0; mode < (quick ? 1 : 2); ++mode) {   // 0: random bf16 values ~N(0,1)-like bit patterns, 1: zeros
         srand(1);
         for (auto &w : h) {
             if (mode == 1) { w = 0; continue; }
@@ -78,17 +82,17 @@ int main(int argc, char **argv) {
             w = rb() | (rb() << 16);
         }
         (void)hipMemcpy(src, h.data(), n * 16, hipMemcpyHostToDevice);
-        for (int which = 0; which < 2; ++which) {
-            const int iters = which == 0 ? 20000 : 10000;   // same flops per launch: 32 x 32768 vs 64 x 16384 per iteration
+        for (int which = 0; which < (quick ? 1 : 2); ++which) {
+            const int iters = (which == 0 ? 20000 : 10000) / (quick ? 8 : 1);   // same flops per launch: 32 x 32768 vs 64 x 16384 per iteration
             const double flops_per_launch = 1024.0 * 4 * (which == 0 ? 32.0 * 32768 : 64.0 * 16384) * iters;
             auto launch = [&] { if (which == 0) hipLaunchKernelGGL(k32, dim3(1024), dim3(256), 0, 0, src, out, iters); else hipLaunchKernelGGL(k16, dim3(1024), dim3(256), 0, 0, src, out, iters); };
             launch(); (void)hipDeviceSynchronize();
             std::atomic<bool> stop{false}; std::vector<double> w; std::vector<int> mhz;
-            std::thread th([&] { while (!stop) { w.push_back(read_num(hwmon + "/power1_input") / 1e6); mhz.push_back(read_sclk()); std::this_thread::sleep_for(std::chrono::milliseconds(200)); } });
+            std::thread th([&] { while (!stop) { w.push_back(read_num(hwmon + "/power1_input") / 1e6); mhz.push_back(read_sclk()); std::this_thread::sleep_for(std::chrono::milliseconds(quick ? 50 : 200)); } });
             hipEvent_t e0, e1; (void)hipEventCreate(&e0); (void)hipEventCreate(&e1);
             auto t0 = std::chrono::steady_clock::now(); int launches = 0;
             (void)hipEventRecord(e0, 0);
-            while (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() < 4.0) { launch(); (void)hipDeviceSynchronize(); ++launches; }
+            while (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() < seconds) { launch(); (void)hipDeviceSynchronize(); ++launches; }
             (void)hipEventRecord(e1, 0); (void)hipEventSynchronize(e1);
             stop = true; th.join();
             float ms; (void)hipEventElapsedTime(&ms, e0, e1);
