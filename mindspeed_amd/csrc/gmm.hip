@@ -391,7 +391,7 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
             for (int i = 0; i < 16; ++i) table->begins[i] = 0x7fffffff;
         }
         return;
-    } else
+    }
     for (int g = g0; g < g1; ++g) {
         const GroupPlan p = plan_of(g);
         const ScanItem it = item_of(p);

@@ -449,11 +449,11 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
         Operand<B_RED, BN> lb;
         la.init(p.a_stride_row, p.a_stride_red, row0, A_RED ? row_end - 1 : row_end - 8, wm * TM * 32);
         if constexpr (SWIGLU) {
-        static_assert(!SWIGLU || !B_RED, "the fused SwiGLU form reads the weight along its columns");
-        lb.init(p.b_stride_col, p.b_stride_red, col0, col_end - 8, wn * TN * 32, col_end - HALF, col_end);
-    } else {
-        lb.init(p.b_stride_col, p.b_stride_red, col0, B_RED ? col_end - 1 : col_end - 8, wn * TN * 32);
-    }
+            static_assert(!SWIGLU || !B_RED, "the fused SwiGLU form reads the weight along its columns");
+            lb.init(p.b_stride_col, p.b_stride_red, col0, col_end - 8, wn * TN * 32, col_end - HALF, col_end);
+        } else {
+            lb.init(p.b_stride_col, p.b_stride_red, col0, B_RED ? col_end - 1 : col_end - 8, wn * TN * 32);
+        }
         // uniform base pointers of element (outer0, red_begin); advanced by one K step per iteration
         const char *a_ptr = static_cast<const char *>(p.a) +
                             (static_cast<int64_t>(row0) * p.a_stride_row + static_cast<int64_t>(red_begin) * p.a_stride_red) * 2;
@@ -468,15 +468,15 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
 
         v16 af[2][TM], bf[2][TN];
         auto read_frags = [&](const char *stage, int set, int kk) {
-    #pragma unroll
+#pragma unroll
             for (int t = 0; t < TM; ++t) af[set][t] = la.frag(stage, kk, t);
-    #pragma unroll
+#pragma unroll
             for (int t = 0; t < TN; ++t) bf[set][t] = lb.frag(stage + A_BYTES, kk, t);
         };
         auto mfmas = [&](int set, int i0, int i1) {
-    #pragma unroll
+#pragma unroll
             for (int i = i0; i < i1; ++i)
-    #pragma unroll
+#pragma unroll
                 for (int j = 0; j < TN; ++j) acc[i][j] = mfma16<DT>(bf[set][j], af[set][i], acc[i][j]);
         };
         // part p of a tile: p = 0,1 -> A halves, p = 2,3 -> B halves
@@ -498,14 +498,14 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
             // tile 0 -> LDS stage 0; tile 1 -> registers.  Both use the masked loads (whose results are
             // consumed at once), so no load is outstanding when the steady-state loop is entered and the
             // loop's own issue order alone decides how long each of its waits has to be.
-    #pragma unroll
+#pragma unroll
             for (int part = 0; part < 4; ++part) load_part(std::true_type{}, part, red_len);
-    #pragma unroll
+#pragma unroll
             for (int part = 0; part < 4; ++part) store_part(lds, part);
             if (nk > 1) {
                 a_ptr += a_step;
                 b_ptr += b_step;
-    #pragma unroll
+#pragma unroll
                 for (int part = 0; part < 4; ++part) load_part(std::true_type{}, part, red_len - BK);
             }
             lds_barrier();
@@ -531,7 +531,7 @@ __device__ __forceinline__ void gmm16_tile(const GmmArgs &p, const TileCoord &tc
                 b_ptr += b_step;
             }
             const int left2 = red_len - (kt + 2) * BK;
-    #pragma unroll
+#pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
                 const int set = kk & 1;
                 if constexpr (HAS1) store_part(nxt, kk);
