@@ -269,6 +269,42 @@ def run_layer(cfg, device, steps, warmup, fuse_activation=False, per_kernel=True
     return ms_per_step, ms_events, kernels, (x, p, idx)
 
 
+def graph_replay_ms(cfg, device, replays=200):
+    """One forward+backward step of the layer recorded into a HIP graph (the C ABI only launches kernels on the
+    caller's stream, so the step can be captured) and replayed: ms per replay, or None if a replay does not reproduce
+    the eager step bit for bit.  For the small configuration, whose eager step time is the host's launch work."""
+    from mindspeed_amd.dispatcher import dispatch_mlp_combine
+
+    x, p, idx, w1, w2, gy = make_inputs(cfg, device)
+
+    def step():
+        leaves = [t.detach().requires_grad_(True) for t in (x, p, w1, w2)]
+        out = dispatch_mlp_combine(leaves[0], idx, leaves[1], (leaves[2], leaves[3]))
+        return (out,) + tuple(torch.autograd.grad(out, leaves, gy))
+
+    eager = [t.clone() for t in step()]
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream(device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph):
+            outs = step()
+    torch.cuda.current_stream(device).wait_stream(side)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    if not all(torch.equal(a, b) for a, b in zip(outs, eager)):
+        return None
+    t0 = time.perf_counter()
+    for _ in range(replays):
+        graph.replay()
+    torch.cuda.synchronize()
+    return round((time.perf_counter() - t0) * 1e3 / replays, 4)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -390,6 +426,8 @@ def main():
                                 "gemm_tflops": {k: ok[k]["tflops"] for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok},
                                 "gemm_frac_of_mfma_peak": {k: ok[k]["frac_of_mfma_peak"]
                                                            for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok}}
+                if name == "plumbing":
+                    others[name]["graph_replay_ms_per_step"] = graph_replay_ms(ocfg, device)
                 torch.cuda.empty_cache()
             # the same Mixtral step with the weight gradients accumulated into fp32 buffers (the reference's
             # gradient-accumulation fusion, mindspeed/ops/gmm.py:56-89) by the product itself, against 16-bit

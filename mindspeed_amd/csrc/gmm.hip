@@ -22,7 +22,7 @@
 //     (element-wise guarded loads, operands that are not contiguous along the
 //     reduction dim transposed in registers on their way to LDS), same
 //     256x256x64 tile and 4x4 v_mfma_f32_32x32x16 per wavefront; and
-//     gmm32_kernel for fp32 inputs (v_mfma_f32_32x32x2f32, 128x128x8 tiles).
+//     gmm32_kernel for fp32 inputs (v_mfma_f32_32x32x2f32, 128x128x16 or 64x64x32 tiles).
 #include <mutex>
 #include <type_traits>
 
@@ -685,83 +685,123 @@ __global__ __launch_bounds__(256) void gmm16_kernel(const GmmArgs p) {
 }
 
 // ---- fp32 MFMA kernel ---------------------------------------------------------------------
-constexpr int FM = 128, FN = 128, FK = 8, FPITCH = 132;
+// v_mfma_f32_32x32x2f32 on square tiles of 64 * TM rows and columns (2 x 2 wavefronts of TM x TM blocks of 32 x 32), K
+// steps of 16 (large tile) or 32 (small tile).  Element-wise guarded loads, so any pair of strides goes.  The next K
+// step's operands are fetched into registers while the current one is multiplied and then written to the other of two
+// LDS buffers: one barrier per step, and the loads have a whole step to arrive.  TM = 2 (128 x 128) for launches with
+// tiles enough for every compute unit, TM = 1 (64 x 64) for small ones, which otherwise leave most of the chip idle.
+constexpr int kTile32Large = 128, kTile32Small = 64;
 
-template <bool ACC>
+template <bool ACC, int TM>
 __global__ __launch_bounds__(256) void gmm32_kernel(const GmmArgs p) {
-    __shared__ float sa[FK][FPITCH];
-    __shared__ float sb[FK][FPITCH];
+    constexpr int T = 64 * TM;
+    constexpr int FK = TM == 1 ? 32 : 16;      // K step: 8 K elements per thread and operand, two 17 KB buffers each
+    constexpr int PITCH = T + 4;
+    constexpr int PER = T * FK / 256;          // elements per thread, operand and K step
+    __shared__ float sa[2][FK][PITCH];
+    __shared__ float sb[2][FK][PITCH];
     const TileCoord tc = locate_tile<false>(p.table);
     if (!tc.valid) return;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int row0 = tc.e.row_begin + tc.row_tile * tc.e.tile_rows;
+    const int row0 = tc.e.row_begin + tc.row_tile * T;
     const int row_end = tc.e.row_end;
-    const int col0 = tc.col_tile * FN;
+    const int col0 = tc.col_tile * T;
     const int col_end = p.cols;
+    const int red_end = tc.e.red_end;
     const float *a_base = static_cast<const float *>(p.a);
     const float *b_base = static_cast<const float *>(p.b) + tc.e.b_off;
     const bool a_red = p.a_stride_red == 1, b_red = p.b_stride_red == 1;
 
-    f32x16 acc[2][2];
+    f32x16 acc[TM][TM];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TM; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    for (int red0 = tc.e.red_begin; red0 < tc.e.red_end; red0 += FK) {
+    // element i of this thread: (reduction index kk, outer index r) inside the tile, consecutive threads along the
+    // operand's contiguous dim
+    auto fetch = [&](float (&ra)[PER], float (&rb)[PER], int red0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < PER; ++i) {
             const int idx = tid + i * 256;
             {
-                const int kk = a_red ? (idx & 7) : (idx >> 7);
-                const int r = a_red ? (idx >> 3) : (idx & 127);
+                const int kk = a_red ? idx % FK : idx / T;
+                const int r = a_red ? idx / FK : idx % T;
                 const int row = row0 + r, red = red0 + kk;
-                sa[kk][r] = (row < row_end && red < tc.e.red_end)
-                                ? a_base[static_cast<int64_t>(row) * p.a_stride_row + static_cast<int64_t>(red) * p.a_stride_red]
-                                : 0.f;
+                ra[i] = (row < row_end && red < red_end)
+                            ? a_base[static_cast<int64_t>(row) * p.a_stride_row + static_cast<int64_t>(red) * p.a_stride_red]
+                            : 0.f;
             }
             {
-                const int kk = b_red ? (idx & 7) : (idx >> 7);
-                const int cc = b_red ? (idx >> 3) : (idx & 127);
+                const int kk = b_red ? idx % FK : idx / T;
+                const int cc = b_red ? idx / FK : idx % T;
                 const int col = col0 + cc, red = red0 + kk;
-                sb[kk][cc] = (col < col_end && red < tc.e.red_end)
-                                 ? b_base[static_cast<int64_t>(red) * p.b_stride_red + static_cast<int64_t>(col) * p.b_stride_col]
-                                 : 0.f;
+                rb[i] = (col < col_end && red < red_end)
+                            ? b_base[static_cast<int64_t>(red) * p.b_stride_red + static_cast<int64_t>(col) * p.b_stride_col]
+                            : 0.f;
             }
         }
-        __syncthreads();
+    };
+    auto stash = [&](int buf, const float (&ra)[PER], const float (&rb)[PER]) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = tid + i * 256;
+            sa[buf][a_red ? idx % FK : idx / T][a_red ? idx / FK : idx % T] = ra[i];
+            sb[buf][b_red ? idx % FK : idx / T][b_red ? idx / FK : idx % T] = rb[i];
+        }
+    };
+    auto multiply = [&](int buf) {
 #pragma unroll
         for (int ks = 0; ks < FK / 2; ++ks) {
             const int kk = ks * 2 + (lane >> 5);
-            float av[2], bv[2];
+            float av[TM], bv[TM];
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                av[t] = sa[kk][wm * 64 + t * 32 + (lane & 31)];
-                bv[t] = sb[kk][wn * 64 + t * 32 + (lane & 31)];
+            for (int t = 0; t < TM; ++t) {
+                av[t] = sa[buf][kk][wm * 32 * TM + t * 32 + (lane & 31)];
+                bv[t] = sb[buf][kk][wn * 32 * TM + t * 32 + (lane & 31)];
             }
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < TM; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[i][j], 0, 0, 0);
         }
-        __syncthreads();
+    };
+
+    // K step t is multiplied out of LDS buffer t & 1 while step t + 1 is fetched into registers, then written to the
+    // other buffer.  (Two steps of fetches in flight instead of one measured the same: at these sizes a step is as long
+    // as its dependent MFMAs.)
+    float ra[PER], rb[PER];
+    const int red_begin = tc.e.red_begin;
+    if (red_begin < red_end) {
+        fetch(ra, rb, red_begin);
+        stash(0, ra, rb);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int red0 = red_begin; red0 < red_end; red0 += FK) {
+        const bool more = red0 + FK < red_end;
+        if (more) fetch(ra, rb, red0 + FK);
+        multiply(buf);
+        if (more) stash(buf ^ 1, ra, rb);
+        __syncthreads();          // everyone is done with `buf`, and the other buffer is complete
+        buf ^= 1;
     }
     float *c_base = static_cast<float *>(p.c) + tc.e.c_off;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int row = row0 + wm * 64 + i * 32 + (lane & 31);
+    for (int i = 0; i < TM; ++i) {
+        const int row = row0 + wm * 32 * TM + i * 32 + (lane & 31);
         if (row >= row_end) continue;
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TM; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int col = col0 + wn * 64 + j * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                const int col = col0 + wn * 32 * TM + j * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                 if (col < col_end) {
                     float *c = c_base + static_cast<int64_t>(row) * p.c_stride_row + col;
                     *c = ACC ? *c + acc[i][j][e] : acc[i][j][e];
@@ -991,8 +1031,13 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     MS_REQUIRE(b_red || b_col, MS_ERR_UNSUPPORTED, "ms_gmm: weight needs one unit stride (got %lld, %lld)", (long long)w_stride0, (long long)w_stride1);
 
     const bool is32 = dtype == MS_FP32;
-    const int tile_rows = is32 ? FM : BM;
-    const int tile_cols = is32 ? FN : BN;
+    const int num_cus = current_device_cus();
+    // fp32: the small tile where the large one would not give every compute unit two tiles
+    const int64_t large32 = (group_type == 0 ? ceil_div(m, kTile32Large) + num_groups / 2 : num_groups * ceil_div(k, kTile32Large)) *
+                            ceil_div(n, kTile32Large);
+    const int tile32 = large32 < 2 * num_cus ? kTile32Small : kTile32Large;
+    const int tile_rows = is32 ? tile32 : BM;
+    const int tile_cols = is32 ? tile32 : BN;
     // fused SwiGLU form: a tile holds 128 gate and the matching 128 up columns, i.e. 128 activation columns
     const int64_t num_col_tiles = swiglu != nullptr ? ceil_div(n / 2, tile_cols / 2) : ceil_div(n, tile_cols);
     const int64_t row_tiles_bound = group_type == 0 ? ceil_div(m, tile_rows) + num_groups + 2
@@ -1002,7 +1047,6 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
 
     TileTable *table = static_cast<TileTable *>(workspace);
     const int64_t c_stride_group = k * y_stride_row;
-    const int num_cus = current_device_cus();
     int64_t *b_offsets = nullptr;
     if (weight_offsets != nullptr) {
         b_offsets = reinterpret_cast<int64_t *>(static_cast<char *>(workspace) + offsets_pos(num_groups));
@@ -1068,10 +1112,13 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     if (is32) {
         MS_REQUIRE(swiglu == nullptr, MS_ERR_UNSUPPORTED, "ms_gmm_swiglu: 16-bit dtypes only");
         if (int rc = schedule(0)) return rc;
-        if (accumulate)
-            hipLaunchKernelGGL(gmm32_kernel<true>, dim3(grid), dim3(256), 0, stream, args);
-        else
-            hipLaunchKernelGGL(gmm32_kernel<false>, dim3(grid), dim3(256), 0, stream, args);
+        if (tile32 == kTile32Large) {
+            if (accumulate) hipLaunchKernelGGL((gmm32_kernel<true, 2>), dim3(grid), dim3(256), 0, stream, args);
+            else hipLaunchKernelGGL((gmm32_kernel<false, 2>), dim3(grid), dim3(256), 0, stream, args);
+        } else {
+            if (accumulate) hipLaunchKernelGGL((gmm32_kernel<true, 1>), dim3(grid), dim3(256), 0, stream, args);
+            else hipLaunchKernelGGL((gmm32_kernel<false, 1>), dim3(grid), dim3(256), 0, stream, args);
+        }
         MS_CHECK_LAUNCH("gmm32_kernel");
         return MS_OK;
     }
