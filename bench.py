@@ -390,12 +390,27 @@ def main():
             _lib.check(lib.ms_copy_bytes(_lib.stream_ptr(device), _lib.ptr(src), _lib.ptr(dst), n), "ms_copy_bytes")
         torch.cuda.synchronize()
         result["copy_calibration_bytes"] = n
-    if not args.no_extras:
+    def extra(name, fn):
+        """Sections beside the headline measurement: one that raises is reported under `extras_failed` and the line
+        is printed all the same."""
+        try:
+            fn()
+        except Exception as exc:      # noqa: BLE001 -- whatever it is, the measured line must still come out
+            import traceback
+            traceback.print_exc(file=sys.stderr)
+            result.setdefault("extras_failed", {})[name] = repr(exc)
+        torch.cuda.empty_cache()
+
+    def probe_section():
         probe = board_mfma_rate()
         if probe is not None:
             result["board_mfma_probe"] = probe
             roofline["frac_of_board_mfma_probe"] = round(dom["tflops"] / probe["tflops"], 4)
+
+    def routing_map_section():
         result["routing_map_mode"] = measure_routing_map_mode(cfg, device, x.detach(), idx, p.detach())
+
+    def permute_family_section():
         # The permute / unpermute family by itself at this workload's shape: back-to-back launches through the C ABI
         # (the per-op figures under "kernels" are single launches inside the layer step, whose operands were last
         # touched hundreds of megabytes of traffic earlier).  "warm": one set of buffers, resident in the 256 MB
@@ -413,35 +428,49 @@ def main():
             "note": "back-to-back launches through the C ABI, event-timed over 200 launches per op; algorithmic bytes "
                     "over the average, against the 8 TB/s HBM peak and against the plain copy kernel in the same mode",
             "cold_buffer_sets": cold_sets, "warm": warm, "cold": cold}
-        # the other two bf16 workloads, forward+backward, 10 steps each after their own warm-up
+
+    others = {}
+
+    def other_workload(name):
+        # forward+backward, 10 steps (50 of the small one) after its own warm-up
+        ocfg = WORKLOADS[name]
+        ms, _, ok, _ = run_layer(ocfg, device, steps=10 if name != "plumbing" else 50, warmup=10)
+        others[name] = {"workload": ocfg["desc"], "ms_per_step": round(ms, 4),
+                        "tokens_per_s": round(ocfg["T"] / (ms / 1e3), 1),
+                        "gemm_tflops": {k: ok[k]["tflops"] for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok},
+                        "gemm_frac_of_mfma_peak": {k: ok[k]["frac_of_mfma_peak"]
+                                                   for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok}}
+
+    def graph_section():
+        others["plumbing"]["graph_replay_ms_per_step"] = graph_replay_ms(WORKLOADS["plumbing"], device)
+
+    def accumulation_section():
+        # the same Mixtral step with the weight gradients accumulated into fp32 buffers (the reference's
+        # gradient-accumulation fusion, mindspeed/ops/gmm.py:56-89) by the product itself, against 16-bit
+        # weight gradients followed by one add each
+        acc = {}
+        for how in ("fused", "separate"):
+            ms, _, ok, _ = run_layer(cfg, device, steps=10, warmup=5, accumulate=how)
+            acc[how] = {"ms_per_step": round(ms, 4),
+                        "gmm_dw_tflops": ok["gmm_dw"]["tflops"] if "gmm_dw" in ok else None}
+            torch.cuda.empty_cache()
+        others["mixtral_fp32_grad_accumulation"] = acc
+
+    if not args.no_extras:
+        extra("board_mfma_probe", probe_section)
+        extra("routing_map_mode", routing_map_section)
+        extra("permute_family", permute_family_section)
         if args.workload == "mixtral":
-            others = {}
             del x, p, idx
             torch.cuda.empty_cache()
             for name in ("deepseek", "qwen", "plumbing"):
-                ocfg = WORKLOADS[name]
-                ms, _, ok, _ = run_layer(ocfg, device, steps=10 if name != "plumbing" else 50, warmup=10)
-                others[name] = {"workload": ocfg["desc"], "ms_per_step": round(ms, 4),
-                                "tokens_per_s": round(ocfg["T"] / (ms / 1e3), 1),
-                                "gemm_tflops": {k: ok[k]["tflops"] for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok},
-                                "gemm_frac_of_mfma_peak": {k: ok[k]["frac_of_mfma_peak"]
-                                                           for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok}}
-                if name == "plumbing":
-                    others[name]["graph_replay_ms_per_step"] = graph_replay_ms(ocfg, device)
-                torch.cuda.empty_cache()
-            # the same Mixtral step with the weight gradients accumulated into fp32 buffers (the reference's
-            # gradient-accumulation fusion, mindspeed/ops/gmm.py:56-89) by the product itself, against 16-bit
-            # weight gradients followed by one add each
-            acc = {}
-            for how in ("fused", "separate"):
-                ms, _, ok, _ = run_layer(cfg, device, steps=10, warmup=5, accumulate=how)
-                acc[how] = {"ms_per_step": round(ms, 4),
-                            "gmm_dw_tflops": ok["gmm_dw"]["tflops"] if "gmm_dw" in ok else None}
-                torch.cuda.empty_cache()
-            others["mixtral_fp32_grad_accumulation"] = acc
+                extra(name, lambda name=name: other_workload(name))
+            if "plumbing" in others:
+                extra("plumbing_graph_replay", graph_section)
+            extra("mixtral_fp32_grad_accumulation", accumulation_section)
             result["other_workloads"] = others
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(cfg)
+        extra("cpu_baseline", lambda: result.__setitem__("cpu_baseline", cpu_baseline(cfg)))
     print(json.dumps(result))
 
 
