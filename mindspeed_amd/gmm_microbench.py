@@ -1,7 +1,7 @@
 """Grouped-matmul launches of the Mixtral-shape expert MLP in isolation.
 
     python -m mindspeed_amd.gmm_microbench [--mode fwd1|fwd2|dx1|dx2|dw1|dw2|dw1acc|dw2acc|library] [--data randn|small|ones|zeros]
-                                           [--counts 988,1074,...] [--iters 20] [--warmup 20]
+                                           [--dtype bf16|fp16|fp32] [--counts 988,1074,...] [--iters 20] [--warmup 20]
 
 ``fwd1`` / ``dx1`` / ``dw1`` are the forward, dX and dW products of the first matmul
 (``[T, H] x [E, H, 2F]``), ``fwd2`` / ``dx2`` / ``dw2`` those of the second (``[T, F] x [E, F, H]``);
@@ -23,6 +23,7 @@ def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--mode", default="fwd1", choices=["fwd1", "fwd2", "dx1", "dx2", "dw1", "dw2", "dw1acc", "dw2acc", "library"])
     ap.add_argument("--data", default="randn", choices=["randn", "small", "ones", "zeros"])
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32"], help="operand dtype")
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--tokens", type=int, default=8192, help="rows after permutation (tokens x top-k)")
@@ -42,7 +43,7 @@ def main():
             raise SystemExit(f"--counts needs {E} entries summing to {T}")
     else:
         counts = torch.full((E,), T // E, dtype=torch.int64, device=dev)
-    bf = torch.bfloat16
+    bf = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[a.dtype]
 
     def operand(*shape):
         if a.data == "zeros":
@@ -90,7 +91,7 @@ def main():
     e1.record()
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / a.iters
-    print(f"{a.mode} ({a.data}): {ms:.4f} ms  {flops / ms / 1e9:.1f} TFLOP/s", flush=True)
+    print(f"{a.mode} ({a.data}{'' if a.dtype == 'bf16' else ', ' + a.dtype}): {ms:.4f} ms  {flops / ms / 1e9:.1f} TFLOP/s", flush=True)
 
 
 if __name__ == "__main__":
