@@ -338,4 +338,138 @@ def _routing_map_probs_grad(row_id_map, grad_permuted_probs, num_tokens, num_exp
 _define("routing_map_probs_grad(Tensor row_id_map, Tensor grad_permuted_probs, int num_tokens, int num_experts) -> Tensor",
         _routing_map_probs_grad, lambda r, g, num_tokens, num_experts: g.new_empty((num_tokens, num_experts)))
 
+
+
+# ---- grouped matmul with one weight matrix per group -----------------------------------------------------------
+def _gmm_weight_list(x, weights, group_list, group_list_type):
+    """``weights``: 2-D ``[K, N]`` views of one shape, dtype and stride pattern (the Python surface has made them so)."""
+    lib = _lib.load()
+    dev = x.device
+    dtype = _lib.dtype_code(x.dtype, "x")
+    num_groups = group_list.numel()
+    m, k = x.shape
+    n = weights[0].size(1)
+    strides = (weights[0].stride(0), weights[0].stride(1))
+    out = torch.empty((m, n), dtype=x.dtype, device=dev)
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(lib.ms_gmm_workspace_size(num_groups, m, 0, ctypes.byref(nbytes)), "ms_gmm_workspace_size")
+    ws = _lib.workspace(nbytes.value, dev)
+    ptrs = (ctypes.c_void_p * num_groups)(*[v.data_ptr() for v in weights])
+    kind = "gmm_dx" if strides[0] == 1 and strides[1] != 1 else "gmm_fwd"
+    with torch.cuda.device(dev), flop_counter.op(kind, flop_counter.gmm_flops(m, k, n), "flop", dev):
+        _lib.check(lib.ms_gmm_weight_list(
+            _lib.stream_ptr(dev), _lib.ptr(x), x.stride(0), x.stride(1), ptrs, strides[0], strides[1], _lib.ptr(out), n,
+            _lib.ptr(group_list), group_list_type, num_groups, m, k, n, dtype, dtype, _lib.ptr(ws), ws.numel()),
+            "ms_gmm_weight_list")
+    return out
+
+
+_define("gmm_weight_list(Tensor x, Tensor[] weights, Tensor group_list, int group_list_type) -> Tensor", _gmm_weight_list,
+        lambda x, weights, group_list, group_list_type: x.new_empty((x.size(0), weights[0].size(1))))
+
+
+# ---- grouped matmul with SwiGLU in its epilogue ------------------------------------------------------------------
+def _gmm_swiglu(x, weight, group_list, group_list_type, probs):
+    """``fc1 = grouped_matmul(x, weight)`` and ``act = silu(gate) * up * probs`` from one launch (contiguous 16-bit
+    operands, checked by the Python surface)."""
+    lib = _lib.load()
+    dev = x.device
+    m, k = x.shape
+    ffn = weight.size(2) // 2
+    p_code = _lib.dtype_code(probs.dtype, "probs") if probs is not None else 0
+    fc1 = torch.empty((m, 2 * ffn), dtype=x.dtype, device=dev)
+    act = torch.empty((m, ffn), dtype=x.dtype, device=dev)
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(lib.ms_gmm_workspace_size(group_list.numel(), m, 0, ctypes.byref(nbytes)), "ms_gmm_workspace_size")
+    ws = _lib.workspace(nbytes.value, dev)
+    with torch.cuda.device(dev), flop_counter.op("gmm_fwd_swiglu", flop_counter.gmm_flops(m, k, 2 * ffn), "flop", dev):
+        _lib.check(lib.ms_gmm_swiglu(
+            _lib.stream_ptr(dev), _lib.ptr(x), x.stride(0), x.stride(1), _lib.ptr(weight), weight.stride(0),
+            weight.stride(1), weight.stride(2), _lib.ptr(fc1), 2 * ffn, _lib.ptr(act), ffn, _lib.ptr(probs), p_code,
+            _lib.ptr(group_list), group_list_type, group_list.numel(), m, k, ffn, _lib.dtype_code(x.dtype, "x"),
+            _lib.ptr(ws), ws.numel()), "ms_gmm_swiglu")
+    return fc1, act
+
+
+_define("gmm_swiglu(Tensor x, Tensor weight, Tensor group_list, int group_list_type, Tensor? probs) -> (Tensor, Tensor)",
+        _gmm_swiglu, lambda x, weight, group_list, group_list_type, probs:
+        (x.new_empty((x.size(0), weight.size(2))), x.new_empty((x.size(0), weight.size(2) // 2))))
+
+
+def _gmm_swiglu_grad(dy, w2, fc1, probs, group_list, group_list_type):
+    """``d_fc1`` (and the probabilities' gradient) from ``dy``: the dX product of the second matmul with the SwiGLU
+    backward on the saved ``fc1`` in its epilogue.  ``w2 [E, ffn, hidden]`` contiguous."""
+    lib = _lib.load()
+    dev = dy.device
+    m, two_ffn = fc1.shape
+    ffn = two_ffn // 2
+    hidden = dy.size(1)
+    num_groups = group_list.numel()
+    d_fc1 = torch.empty_like(fc1)
+    gp = torch.empty_like(probs) if probs is not None else torch.empty(0, dtype=fc1.dtype, device=dev)
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(lib.ms_gmm_swiglu_grad_workspace_size(num_groups, m, ffn, ctypes.byref(nbytes)),
+               "ms_gmm_swiglu_grad_workspace_size")
+    ws = _lib.workspace(nbytes.value, dev)
+    wt = w2.transpose(1, 2)       # [E, hidden, ffn] view: element (k, n) of group g is w2[g, n, k]
+    with torch.cuda.device(dev), flop_counter.op("gmm_dx_swiglu", flop_counter.gmm_flops(m, hidden, ffn), "flop", dev):
+        _lib.check(lib.ms_gmm_swiglu_grad(
+            _lib.stream_ptr(dev), _lib.ptr(dy), dy.stride(0), dy.stride(1), _lib.ptr(w2), wt.stride(0),
+            wt.stride(1), wt.stride(2), _lib.ptr(fc1), two_ffn, _lib.ptr(probs),
+            _lib.dtype_code(probs.dtype, "probs") if probs is not None else 0, _lib.ptr(d_fc1), two_ffn,
+            _lib.ptr(gp) if probs is not None else None, _lib.ptr(group_list), group_list_type, num_groups, m, hidden,
+            ffn, _lib.dtype_code(dy.dtype, "grad"), _lib.ptr(ws), ws.numel()), "ms_gmm_swiglu_grad")
+    return d_fc1, gp
+
+
+_define("gmm_swiglu_grad(Tensor dy, Tensor w2, Tensor fc1, Tensor? probs, Tensor group_list, int group_list_type) "
+        "-> (Tensor, Tensor)", _gmm_swiglu_grad,
+        lambda dy, w2, fc1, probs, group_list, group_list_type:
+        (torch.empty_like(fc1), torch.empty_like(probs) if probs is not None else fc1.new_empty(0)))
+
+
+# ---- chunk sort ------------------------------------------------------------------------------------------------------
+def _sort_chunks(inp, split_sizes, sorted_idxs, probs, zero_fill):
+    """Rows of ``inp`` (and entries of ``probs``) regrouped chunk by chunk, and the row map for the way back.
+    ``zero_fill``: the outputs start as zeros (chunk lists that could not be checked on the host)."""
+    lib = _lib.load()
+    dev = inp.device
+    rows, hidden = inp.shape
+    new = torch.zeros_like if zero_fill else torch.empty_like
+    out = new(inp)
+    row_map = torch.empty(rows, dtype=torch.int32, device=dev)
+    out_p = new(probs) if probs is not None else torch.empty(0, dtype=inp.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.ms_sort_chunks(
+            _lib.stream_ptr(dev), _lib.ptr(inp), _lib.ptr(split_sizes), _lib.ptr(sorted_idxs),
+            split_sizes.numel(), rows, hidden, _lib.dtype_code(inp.dtype, "input"), _lib.ptr(probs),
+            _lib.dtype_code(probs.dtype, "probs") if probs is not None else 0, _lib.ptr(out),
+            _lib.ptr(out_p) if probs is not None else None, _lib.ptr(row_map)), "ms_sort_chunks")
+    return out, out_p, row_map
+
+
+_define("sort_chunks(Tensor input, Tensor split_sizes, Tensor sorted_idxs, Tensor? probs, bool zero_fill) "
+        "-> (Tensor, Tensor, Tensor)", _sort_chunks,
+        lambda inp, split_sizes, sorted_idxs, probs, zero_fill:
+        (torch.empty_like(inp), torch.empty_like(probs) if probs is not None else inp.new_empty(0),
+         inp.new_empty((inp.size(0),), dtype=torch.int32)))
+
+
+def _gather_rows(src, row_map, zero_fill):
+    """``out[row_map[i]] = src[i]`` over the rows of a matrix or the entries of a vector (the chunk sort's way back)."""
+    lib = _lib.load()
+    dev = src.device
+    out = torch.zeros_like(src) if zero_fill else torch.empty_like(src)
+    rows = src.size(0)
+    width = src.size(1) if src.dim() == 2 else 1
+    with torch.cuda.device(dev):
+        _lib.check(lib.ms_gather_rows(_lib.stream_ptr(dev), _lib.ptr(src), _lib.ptr(row_map), rows, width,
+                                      _lib.dtype_code(src.dtype, "grad"), 1, _lib.ptr(out)), "ms_gather_rows")
+    return out
+
+
+_define("gather_rows(Tensor src, Tensor row_map, bool zero_fill) -> Tensor", _gather_rows,
+        lambda src, row_map, zero_fill: torch.empty_like(src))
+
+
 K = torch.ops.mindspeed_amd

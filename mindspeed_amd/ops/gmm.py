@@ -98,13 +98,12 @@ def gmm_raw_weight_list(x, weights, group_list, group_list_type, transposed=Fals
     ``weights``: sequence of 2-D tensors of one shape, dtype and stride pattern; ``W_g = weights[g]``
     (``[K, N]``), or ``weights[g].T`` with ``transposed`` (``[N, K]`` parameters read in place).
     """
-    lib = _lib.load()
     _lib.require_device(x, "x")
     weights = list(weights)
     if not weights:
         raise RuntimeError("Neither x nor weight could be empty")
     dev = x.device
-    dtype = _lib.dtype_code(x.dtype, "x")
+    _lib.dtype_code(x.dtype, "x")
     x = _unit_stride_view(x)
     first = weights[0]
     views = []
@@ -129,20 +128,7 @@ def gmm_raw_weight_list(x, weights, group_list, group_list_type, transposed=Fals
     if x.dim() != 2 or len(views) != num_groups or views[0].size(0) != x.size(1):
         raise ValueError(f"{len(views)} weights of shape {tuple(views[0].shape)} do not match x {tuple(x.shape)} "
                          f"and {num_groups} groups")
-    m, k = x.shape
-    n = views[0].size(1)
-    out = torch.empty((m, n), dtype=x.dtype, device=dev)
-    nbytes = ctypes.c_size_t(0)
-    _lib.check(lib.ms_gmm_workspace_size(num_groups, m, 0, ctypes.byref(nbytes)), "ms_gmm_workspace_size")
-    ws = _lib.workspace(nbytes.value, dev)
-    ptrs = (ctypes.c_void_p * num_groups)(*[v.data_ptr() for v in views])
-    kind = "gmm_dx" if strides[0] == 1 and strides[1] != 1 else "gmm_fwd"
-    with torch.cuda.device(dev), flop_counter.op(kind, flop_counter.gmm_flops(m, k, n), "flop", dev):
-        _lib.check(lib.ms_gmm_weight_list(
-            _lib.stream_ptr(dev), _lib.ptr(x), x.stride(0), x.stride(1), ptrs, strides[0], strides[1], _lib.ptr(out), n,
-            _lib.ptr(gl), group_list_type, num_groups, m, k, n, dtype, dtype, _lib.ptr(ws), ws.numel()),
-            "ms_gmm_weight_list")
-    return out
+    return K.gmm_weight_list(x, views, gl, group_list_type)
 
 
 # dX and dW of one grouped matmul are independent; each is a full-chip kernel whose last round of tiles may leave

@@ -16,18 +16,16 @@ not saved for backward (nothing in this function's backward needs it).
 """
 from __future__ import annotations
 
-import ctypes
-
 import torch
 
-from .. import _lib, flop_counter
+from .. import _lib
+from ._kernels import K
 from .gmm import _beside, _group_list_tensor, gmm_raw
 
 __all__ = ["gmm_swiglu", "GmmSwigluFunction", "grouped_mlp", "GroupedMLPFunction"]
 
 
 def _gmm_swiglu_forward(x, weight, group_list, group_list_type, probs):
-    lib = _lib.load()
     _lib.require_device(x, "x")
     _lib.require_device(weight, "weight")
     if x.dim() != 2 or weight.dim() != 3 or weight.size(1) != x.size(1) or weight.size(2) % 2 != 0:
@@ -42,27 +40,15 @@ def _gmm_swiglu_forward(x, weight, group_list, group_list_type, probs):
     gl = _group_list_tensor(group_list, dev)
     if gl.dtype != torch.int64 or gl.dim() != 1 or gl.numel() != weight.size(0):
         raise TypeError("group_list must be a one-dimensional int64 tensor with one entry per expert")
-    m, k = x.shape
-    ffn = weight.size(2) // 2
+    m = x.size(0)
     p = None
-    p_code = 0
     if probs is not None:
         _lib.require_device(probs, "probs")
         p = probs.contiguous().view(-1)
         if p.numel() != m:
             raise RuntimeError(f"probs has {p.numel()} entries, expected {m}")
-        p_code = _lib.dtype_code(p.dtype, "probs")
-    fc1 = torch.empty((m, 2 * ffn), dtype=x.dtype, device=dev)
-    act = torch.empty((m, ffn), dtype=x.dtype, device=dev)
-    nbytes = ctypes.c_size_t(0)
-    _lib.check(lib.ms_gmm_workspace_size(gl.numel(), m, 0, ctypes.byref(nbytes)), "ms_gmm_workspace_size")
-    ws = _lib.workspace(nbytes.value, dev)
-    with torch.cuda.device(dev), flop_counter.op("gmm_fwd_swiglu", flop_counter.gmm_flops(m, k, 2 * ffn), "flop", dev):
-        _lib.check(lib.ms_gmm_swiglu(
-            _lib.stream_ptr(dev), _lib.ptr(x), x.stride(0), x.stride(1), _lib.ptr(weight), weight.stride(0),
-            weight.stride(1), weight.stride(2), _lib.ptr(fc1), 2 * ffn, _lib.ptr(act), ffn, _lib.ptr(p), p_code,
-            _lib.ptr(gl), group_list_type, gl.numel(), m, k, ffn, _lib.dtype_code(x.dtype, "x"), _lib.ptr(ws),
-            ws.numel()), "ms_gmm_swiglu")
+        _lib.dtype_code(p.dtype, "probs")
+    fc1, act = K.gmm_swiglu(x, weight, gl, group_list_type, p)
     return fc1, act, gl, p
 
 
@@ -78,19 +64,8 @@ class GmmSwigluFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_act):
         x, weight, gl, fc1, p = ctx.saved_tensors
-        lib = _lib.load()
         dev = grad_act.device
-        rows, two_ffn = fc1.shape
-        ffn = two_ffn // 2
-        g = grad_act.contiguous()
-        d_fc1 = torch.empty_like(fc1)
-        gp = torch.empty_like(p) if p is not None else None
-        p_code = _lib.dtype_code(p.dtype, "probs") if p is not None else 0
-        with torch.cuda.device(dev), flop_counter.op(
-                "swiglu_grad", flop_counter.swiglu_bytes(rows, ffn, fc1.element_size(), True), "byte", dev):
-            _lib.check(lib.ms_swiglu_grad(_lib.stream_ptr(dev), _lib.ptr(g), _lib.ptr(fc1), _lib.ptr(p), p_code, rows,
-                                          ffn, _lib.dtype_code(fc1.dtype, "x"), _lib.ptr(d_fc1), _lib.ptr(gp)),
-                       "ms_swiglu_grad")
+        d_fc1, gp = _swiglu_grad_from_fc1(grad_act.contiguous(), fc1, p)
         glt = ctx.group_list_type
         dx = dw = None
         if ctx.needs_input_grad[1]:
@@ -119,31 +94,12 @@ def gmm_swiglu(x, weight, group_list, probs=None, *, group_list_type: int = 1):
 
 def _swiglu_from_fc1(fc1, p):
     """The activation again from the saved fc1 output (the recomputation of experts.py:183-191)."""
-    lib = _lib.load()
-    rows, two_ffn = fc1.shape
-    ffn = two_ffn // 2
-    act = torch.empty((rows, ffn), dtype=fc1.dtype, device=fc1.device)
-    with torch.cuda.device(fc1.device), flop_counter.op(
-            "swiglu", flop_counter.swiglu_bytes(rows, ffn, fc1.element_size()), "byte", fc1.device):
-        _lib.check(lib.ms_swiglu(_lib.stream_ptr(fc1.device), _lib.ptr(fc1), _lib.ptr(p),
-                                 _lib.dtype_code(p.dtype, "probs") if p is not None else 0, rows, ffn,
-                                 _lib.dtype_code(fc1.dtype, "x"), _lib.ptr(act)), "ms_swiglu")
-    return act
+    return K.swiglu(fc1, p)
 
 
 def _swiglu_grad_from_fc1(dact, fc1, p):
-    lib = _lib.load()
-    rows, two_ffn = fc1.shape
-    ffn = two_ffn // 2
-    dev = fc1.device
-    d_fc1 = torch.empty_like(fc1)
-    gp = torch.empty_like(p) if p is not None else None
-    with torch.cuda.device(dev), flop_counter.op(
-            "swiglu_grad", flop_counter.swiglu_bytes(rows, ffn, fc1.element_size(), True), "byte", dev):
-        _lib.check(lib.ms_swiglu_grad(_lib.stream_ptr(dev), _lib.ptr(dact), _lib.ptr(fc1), _lib.ptr(p),
-                                      _lib.dtype_code(p.dtype, "probs") if p is not None else 0, rows, ffn,
-                                      _lib.dtype_code(fc1.dtype, "x"), _lib.ptr(d_fc1), _lib.ptr(gp)), "ms_swiglu_grad")
-    return d_fc1, gp
+    d_fc1, gp = K.swiglu_grad(dact, fc1, p)
+    return d_fc1, (gp if p is not None else None)
 
 
 class GroupedMLPFunction(torch.autograd.Function):
@@ -191,14 +147,9 @@ class GroupedMLPFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         x, w1, w2, gl, fc1, p, act = ctx.saved_tensors
-        lib = _lib.load()
         dev = grad_out.device
         glt = ctx.group_list_type
         dy = grad_out.contiguous()
-        m, two_ffn = fc1.shape
-        ffn = two_ffn // 2
-        hidden = dy.size(1)
-        num_groups = gl.numel()
         if act is None:
             act = _swiglu_from_fc1(fc1, p)
         # everything the side stream writes is allocated here, on the caller's stream
@@ -209,22 +160,8 @@ class GroupedMLPFunction(torch.autograd.Function):
             if dw2 is not None:
                 gmm_raw(act.t(), dy, gl, 2, glt, out=dw2)
         if ctx.fused_kernels:
-            w2c = w2.contiguous()
-            d_fc1 = torch.empty_like(fc1)
-            gp = torch.empty_like(p) if p is not None else None
-            nbytes = ctypes.c_size_t(0)
-            _lib.check(lib.ms_gmm_swiglu_grad_workspace_size(num_groups, m, ffn, ctypes.byref(nbytes)),
-                       "ms_gmm_swiglu_grad_workspace_size")
-            ws = _lib.workspace(nbytes.value, dev)
-            wt = w2c.transpose(1, 2)       # [E, hidden, ffn] view: element (k, n) of group g is w2[g, n, k]
-            with torch.cuda.device(dev), flop_counter.op("gmm_dx_swiglu", flop_counter.gmm_flops(m, hidden, ffn),
-                                                         "flop", dev):
-                _lib.check(lib.ms_gmm_swiglu_grad(
-                    _lib.stream_ptr(dev), _lib.ptr(dy), dy.stride(0), dy.stride(1), _lib.ptr(w2c), wt.stride(0),
-                    wt.stride(1), wt.stride(2), _lib.ptr(fc1), two_ffn, _lib.ptr(p),
-                    _lib.dtype_code(p.dtype, "probs") if p is not None else 0, _lib.ptr(d_fc1), two_ffn, _lib.ptr(gp),
-                    _lib.ptr(gl), glt, num_groups, m, hidden, ffn, _lib.dtype_code(dy.dtype, "grad"), _lib.ptr(ws),
-                    ws.numel()), "ms_gmm_swiglu_grad")
+            d_fc1, gp = K.gmm_swiglu_grad(dy, w2.contiguous(), fc1, p, gl, glt)
+            gp = gp if p is not None else None
         else:
             dact = gmm_raw(dy, w2.transpose(1, 2), gl, 0, glt)
             d_fc1, gp = _swiglu_grad_from_fc1(dact, fc1, p)

@@ -16,6 +16,7 @@ from __future__ import annotations
 import torch
 
 from .. import _lib
+from ._kernels import K
 
 __all__ = ["sort_chunks_by_idxs"]
 
@@ -29,27 +30,16 @@ def _as_i64(v, device):
 class _SortChunks(torch.autograd.Function):
     @staticmethod
     def forward(ctx, inp, split_sizes, sorted_idxs, probs, checked):
-        lib = _lib.load()
-        new = torch.empty_like if checked else torch.zeros_like
         ctx.checked = checked
         _lib.require_device(inp, "input")
         if inp.dim() != 2:
             raise RuntimeError(f"input must be 2 dimensional, got {inp.dim()}-dimensional")
         inp = inp.contiguous()
-        dev = inp.device
-        rows, hidden = inp.shape
-        out = new(inp)
-        row_map = torch.empty(rows, dtype=torch.int32, device=dev)
+        rows = inp.size(0)
         p = probs.contiguous() if probs is not None else None
-        out_p = new(p) if p is not None else None
         if p is not None and p.numel() != rows:
             raise RuntimeError(f"probs has {p.numel()} entries, expected {rows}")
-        with torch.cuda.device(dev):
-            _lib.check(lib.ms_sort_chunks(
-                _lib.stream_ptr(dev), _lib.ptr(inp), _lib.ptr(split_sizes), _lib.ptr(sorted_idxs),
-                split_sizes.numel(), rows, hidden, _lib.dtype_code(inp.dtype, "input"), _lib.ptr(p),
-                _lib.dtype_code(p.dtype, "probs") if p is not None else 0, _lib.ptr(out), _lib.ptr(out_p),
-                _lib.ptr(row_map)), "ms_sort_chunks")
+        out, out_p, row_map = K.sort_chunks(inp, split_sizes, sorted_idxs, p, not checked)
         ctx.save_for_backward(row_map)
         ctx.set_materialize_grads(False)
         ctx.has_probs = p is not None
@@ -63,22 +53,10 @@ class _SortChunks(torch.autograd.Function):
         (row_map,) = ctx.saved_tensors
         if grad_out is None:
             return None, None, None, None, None
-        lib = _lib.load()
-        new = torch.empty_like if ctx.checked else torch.zeros_like
-        dev = grad_out.device
-        g = grad_out.contiguous()
-        gi = new(g)
-        with torch.cuda.device(dev):
-            _lib.check(lib.ms_gather_rows(_lib.stream_ptr(dev), _lib.ptr(g), _lib.ptr(row_map), g.size(0), g.size(1),
-                                          _lib.dtype_code(g.dtype, "grad"), 1, _lib.ptr(gi)), "ms_gather_rows")
+        gi = K.gather_rows(grad_out.contiguous(), row_map, not ctx.checked)
         gp = None
         if ctx.has_probs and grad_probs is not None:
-            gpc = grad_probs.contiguous()
-            gp = new(gpc)
-            with torch.cuda.device(dev):
-                _lib.check(lib.ms_gather_rows(_lib.stream_ptr(dev), _lib.ptr(gpc), _lib.ptr(row_map), gpc.numel(), 1,
-                                              _lib.dtype_code(gpc.dtype, "grad_probs"), 1, _lib.ptr(gp)),
-                           "ms_gather_rows")
+            gp = K.gather_rows(grad_probs.contiguous(), row_map, not ctx.checked)
         return gi, None, None, gp, None
 
 

@@ -139,9 +139,11 @@ def test_zero_tokens_give_zero_weight_gradients(dtype, device):
     assert torch.count_nonzero(mlp.weight1.grad) == 0 and torch.count_nonzero(mlp.weight2.grad) == 0
 
 
-def test_layer_traced_by_torch_compile(device):
-    """``torch.compile`` (AOT-traced, eager kernels) of the whole layer, forward and backward: the trace goes through
-    the ops' fake kernels, the run through the same HIP kernels, so results equal the eager ones bit for bit."""
+@pytest.mark.parametrize("fuse", [False, True])
+def test_layer_traced_by_torch_compile(fuse, device):
+    """``torch.compile`` (AOT-traced, eager kernels) of the whole layer, forward and backward, with one kernel per op
+    and with the SwiGLU passes fused into the grouped matmuls: the trace goes through the ops' fake kernels, the run
+    through the same HIP kernels, so results equal the eager ones bit for bit."""
     gen = torch.Generator().manual_seed(34)
     T, H, E, K, F, dtype = 256, 128, 8, 2, 96, torch.bfloat16
     x = torch.randn(T, H, generator=gen).to(dtype).to(device)
@@ -152,7 +154,7 @@ def test_layer_traced_by_torch_compile(device):
     gy = torch.randn(T, H, generator=gen).to(dtype).to(device)
 
     def layer(x, p, w1, w2):
-        return dispatch_mlp_combine(x, idx, p, (w1, w2))
+        return dispatch_mlp_combine(x, idx, p, (w1, w2), fuse_activation=fuse)
 
     def run(fn):
         leaves = [t.clone().requires_grad_(True) for t in (x, p, w1, w2)]

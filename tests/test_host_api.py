@@ -235,6 +235,32 @@ def test_shapes_propagate_on_meta_tensors():
     back.sum().backward()
     assert mprobs.grad.shape == (T, E)
 
+    # the fused matmul + SwiGLU forms, the one-parameter-per-expert module and the chunk sort
+    from mindspeed_amd.ops.gmm_swiglu import gmm_swiglu, grouped_mlp
+    xs, rp = meta(T * K, H, grad=True), meta(T * K, dtype=torch.float32, grad=True)
+    act = gmm_swiglu(xs, w1, gl, rp)
+    assert act.shape == (T * K, F) and act.dtype == torch.bfloat16
+    act.sum().backward()
+    assert xs.grad.shape == xs.shape and rp.grad.shape == rp.shape
+    for fused in (True, False):
+        for recompute in (False, True):
+            xm = meta(T * K, H, grad=True)
+            out = grouped_mlp(xm, w1, w2, gl, rp, recompute_activation=recompute, fused_kernels=fused)
+            assert out.shape == (T * K, H)
+            out.sum().backward()
+            assert xm.grad.shape == xm.shape
+    layer = ops.MindSpeedTEGroupedLinear(E, H, 24, params_dtype=torch.bfloat16, device="meta")
+    xl = meta(T * K, H, grad=True)
+    yl, bias = layer(xl, [32, 32, 32, 32])
+    assert yl.shape == (T * K, 24) and bias is None
+    yl.sum().backward()
+    assert xl.grad.shape == xl.shape and all(p.grad.shape == (24, H) for p in layer.total_weight)
+    xc, pc = meta(T, H, grad=True), meta(T, dtype=torch.float32, grad=True)
+    oc, opc = ops.sort_chunks_by_idxs(xc, meta(4, dtype=torch.int64), meta(4, dtype=torch.int64), pc)
+    assert oc.shape == (T, H) and opc.shape == (T,)
+    (oc.sum() + opc.sum()).backward()
+    assert xc.grad.shape == (T, H) and pc.grad.shape == (T,)
+
 
 def test_probe_sources_and_trace_build_are_wired():
     """The hardware probes are listed by their runner, and the diagnostic (tile trace) build has its own output path."""
