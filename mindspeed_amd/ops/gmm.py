@@ -186,6 +186,25 @@ class _beside:
             self.main.wait_stream(self.side)
 
 
+def _add_group_bias(y, bias, group_list, group_list_type):
+    """``y[rows of group g] += bias[g]`` (forward only, as in the reference: mindspeed/ops/gmm.py:27-28 refuses a bias
+    that requires a gradient).  ``bias [E, N]``, fp16 / bf16 / fp32.  Plain torch ops on the device, nothing read
+    back: the sum is formed in fp32 from the product as the grouped matmul stored it and rounded once more, rows past
+    the last offset stay zero.  How the vendor kernel rounds (it may add before its only rounding) is not stated in the
+    reference tree."""
+    _lib.require_device(bias, "bias")
+    gl = _group_list_tensor(group_list, y.device)
+    num_groups = gl.numel()
+    if bias.dim() != 2 or bias.size(0) != num_groups or bias.size(1) != y.size(1):
+        raise ValueError(f"bias must be [{num_groups}, {y.size(1)}], got {tuple(bias.shape)}")
+    ends = gl if group_list_type == 0 else torch.cumsum(gl, dim=0)
+    rows = torch.arange(y.size(0), device=y.device)
+    group = torch.searchsorted(ends, rows, right=True)
+    covered = (group < num_groups).unsqueeze(1)
+    picked = bias.index_select(0, group.clamp(max=num_groups - 1)).float()
+    return torch.where(covered, y.float() + picked, y.float()).to(y.dtype)
+
+
 class _RawGmmModule:
     """Stand-in for the pybind module of mindspeed/ops/csrc/cann/gmm.cpp:295-309.
 
@@ -196,12 +215,15 @@ class _RawGmmModule:
 
     @staticmethod
     def npu_gmm(x, weight, bias, group_list, group_type, group_list_type):
-        if bias:
-            raise ValueError("bias is not supported by the grouped matmul kernels")
         if len(x) != 1 or len(weight) != 1:
             raise RuntimeError("Neither x nor weight could be empty; single-tensor (split_item=3) form only.")
-        return [gmm_raw(x[0], weight[0], group_list, group_type if group_type is not None else 0,
-                        group_list_type or 0)]
+        group_type = group_type if group_type is not None else 0
+        y = gmm_raw(x[0], weight[0], group_list, group_type, group_list_type or 0)
+        if bias:
+            if len(bias) != 1 or group_type != 0:
+                raise ValueError("bias: one [E, N] tensor, with the split on rows (group_type 0) only")
+            y = _add_group_bias(y, bias[0], group_list, group_list_type or 0)
+        return [y]
 
     @staticmethod
     def npu_gmm_backward(grad, x, weight, group_list, group_list_type):
@@ -389,8 +411,8 @@ def _npu_gmm_common(original_weight, x, weight, *, bias=None, group_list=None, g
                                group_list_type=group_list_type)
     if group_list is None:
         raise ValueError("group_list is required: the single-tensor (split_item=3) form needs group boundaries")
-    if bias is not None:
-        raise ValueError("bias is not supported by the grouped matmul kernels")
+    if bias is not None and group_type != 0:
+        raise ValueError("bias is supported with the split on rows (group_type 0) only")
     if group_list_type == 0:
         return torch.ops.mindspeed.npu_gmm(original_weight, x, weight, bias=bias, group_list=group_list,
                                            group_type=group_type, gemm_fusion=gemm_fusion)

@@ -261,6 +261,40 @@ def test_groupmatmul_add_many_groups(device):
     assert rel_l2(acc, O.groupmatmul_add_fp32(x, dy, offsets, acc0.clone())) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_forward_bias(dtype, device):
+    """``bias [E, N]`` is added to every row of its group in the forward pass (docs/zh/ops/gmm.md: forward only; a
+    bias that requires a gradient is refused, mindspeed/ops/gmm.py:27-28); rows past the last offset stay zero, and
+    the gradients of x and weight are what they are without it."""
+    say("forward bias", dtype)
+    gen = torch.Generator().manual_seed(17)
+    counts = [130, 0, 300, 77, 1, 64]
+    M, K, N, E, extra = sum(counts), 96, 160, len(counts), 9
+    x = torch.randn(M + extra, K, generator=gen).to(dtype)
+    w = (torch.randn(E, K, N, generator=gen) * 0.1).to(dtype)
+    bias = torch.randn(E, N, generator=gen).to(torch.float32 if dtype == torch.bfloat16 else dtype)
+    cum = torch.cumsum(torch.tensor(counts), 0)
+    exp = torch.zeros(M + extra, N, dtype=torch.float64)
+    exp[:M] = O.grouped_matmul(x[:M].double(), counts, w.double()) + torch.repeat_interleave(bias.double(), torch.tensor(counts), dim=0)
+    xd, wd = x.to(device).requires_grad_(True), w.to(device).requires_grad_(True)
+    for y in (ops.npu_gmm(xd, wd, bias=bias.to(device), group_list=cum.tolist(), group_type=0),
+              ops.npu_gmm(xd, wd, bias=bias.to(device), group_list=cum.to(device), group_type=0),
+              ops.npu_gmm_v2(xd, wd, bias=bias.to(device), group_list=torch.tensor(counts, device=device), group_type=0)):
+        assert y.dtype == dtype and rel_l2(y, exp) <= TOL[dtype]
+        assert torch.count_nonzero(y[M:]) == 0
+    gy = torch.randn(M + extra, N, generator=gen).to(dtype)
+    y.backward(gy.to(device))
+    e_dx, e_dw = O.gmm_backward(gy[:M], x[:M], w, counts, 1)
+    assert rel_l2(xd.grad[:M], e_dx) <= TOL[dtype] and rel_l2(wd.grad, e_dw) <= TOL[dtype]
+    with pytest.raises(ValueError, match="gradient"):
+        ops.npu_gmm(xd, wd, bias=bias.to(device).requires_grad_(True), group_list=cum.tolist(), group_type=0)
+    with pytest.raises(ValueError, match="bias"):
+        ops.npu_gmm(xd.detach().t()[:, :M], torch.randn(M, N).to(dtype).to(device), bias=bias.to(device),
+                    group_list=cum.tolist(), group_type=2)
+    with pytest.raises(ValueError, match="bias must be"):
+        ops.npu_gmm(xd, wd, bias=bias[:, :8].to(device), group_list=cum.tolist(), group_type=0)
+
+
 def test_linearity_at_mixtral_fc1_shape(device):
     """Full-size property check on the Mixtral fc1 shape: gmm(a*x1 + x2) == a*gmm(x1) + gmm(x2) within bf16
     rounding, and sampled rows against per-row fp32 matmuls."""
