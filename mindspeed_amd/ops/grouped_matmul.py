@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import torch
 
-from .gmm import gmm_raw
+from .gmm import _add_group_bias, gmm_raw
 
 __all__ = ["_GroupedMatmul", "fused_grouped_matmul"]
 
@@ -19,8 +19,6 @@ __all__ = ["_GroupedMatmul", "fused_grouped_matmul"]
 class _GroupedMatmul(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input_tensor: torch.Tensor, weights, weights_bias, m_split, group_list_type) -> torch.Tensor:
-        if weights_bias is not None:
-            raise ValueError("bias is not supported by the grouped matmul kernels")
         if not isinstance(m_split, torch.Tensor):   # grouped_matmul.py:13-17
             m_split = torch.tensor(list(m_split), device=input_tensor.device, dtype=torch.int64)
         ctx.group_list = m_split
@@ -31,7 +29,13 @@ class _GroupedMatmul(torch.autograd.Function):
         ctx.needs_transpose = weights.shape[1] != input_tensor.shape[-1]
         ctx.save_for_backward(input_tensor, weights)
         w = weights.transpose(1, 2) if ctx.needs_transpose else weights
-        return gmm_raw(input_tensor, w, ctx.group_list, 0, group_list_type)
+        out = gmm_raw(input_tensor, w, ctx.group_list, 0, group_list_type)
+        if weights_bias is not None:
+            # grouped_matmul.py:40-42 hands `weights_bias` to the vendor op beside the list of weight slices: one [N]
+            # vector per group (a stacked [E, N] tensor is taken too); no gradient flows to it (:80 returns None)
+            bias = weights_bias if isinstance(weights_bias, torch.Tensor) else torch.stack(list(weights_bias))
+            out = _add_group_bias(out, bias, ctx.group_list, group_list_type)
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):

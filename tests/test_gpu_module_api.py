@@ -95,6 +95,26 @@ def test_te_grouped_linear(counts, K, N, dtype, device):
             assert rel_l2(p.grad.t(), exp_dw[i]) <= TOL[dtype]
 
 
+def test_stacked_weights_with_bias(device):
+    """``_GroupedMatmul`` with per-group bias vectors (the argument that mindspeed/ops/grouped_matmul.py:40-42 passes
+    on to the vendor op), as a list and stacked; the bias gets no gradient."""
+    counts, K, N, dtype = [130, 0, 300, 77], 64, 96, torch.bfloat16
+    say("stacked weights with bias", counts)
+    E, M = len(counts), sum(counts)
+    gen = torch.Generator().manual_seed(11)
+    x = torch.randn(M, K, generator=gen).to(dtype)
+    w = (torch.randn(E, K, N, generator=gen) * 0.1).to(dtype)
+    bias = torch.randn(E, N, generator=gen).to(dtype)
+    exp = O.grouped_matmul(x.double(), counts, w.double()) + torch.repeat_interleave(bias.double(), torch.tensor(counts), dim=0)
+    xd, wd = x.to(device).requires_grad_(True), w.to(device).requires_grad_(True)
+    bias_list = [b.to(device) for b in bias]
+    out = ops._GroupedMatmul.apply(xd, wd, bias_list, counts, 1)
+    out2 = ops._GroupedMatmul.apply(xd, wd, bias.to(device), torch.tensor(counts, device=device), 1)
+    assert rel_l2(out, exp) <= TOL[dtype] and torch.equal(out, out2)
+    out.sum().backward()
+    assert xd.grad.shape == x.shape and wd.grad.shape == w.shape
+
+
 def test_weight_list_limits(device):
     from mindspeed_amd.ops.gmm import gmm_raw_weight_list
     x = torch.randn(8, 16, device=device)

@@ -151,8 +151,8 @@ def test_routing_map_and_module_api_surface():
         ops.fused_grouped_matmul(x, [4, 4], torch.randn(2, 16, 4, dtype=torch.bfloat16))
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         ops.MindSpeedTEGroupedLinear(2, 16, 4, params_dtype=torch.bfloat16)(x, [4, 4])
-    with pytest.raises(ValueError, match="bias"):
-        ops._GroupedMatmul.apply(x, torch.randn(2, 16, 4, dtype=torch.bfloat16), torch.zeros(4), [4, 4], 1)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops._GroupedMatmul.apply(x, torch.randn(2, 16, 4, dtype=torch.bfloat16), torch.zeros(2, 4), [4, 4], 1)
 
 
 def test_fused_mlp_argument_checks():
