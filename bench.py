@@ -269,6 +269,24 @@ def run_layer(cfg, device, steps, warmup, fuse_activation=False, per_kernel=True
     return ms_per_step, ms_events, kernels, (x, p, idx)
 
 
+def forward_only_ms(cfg, device, fuse_activation, steps=20, warmup=10):
+    """The layer's forward pass alone under ``torch.no_grad()`` (inference): ms per pass.  With ``fuse_activation`` the
+    SwiGLU comes out of the first grouped matmul's epilogue and the fc1 output, which only a backward pass would read,
+    is not stored."""
+    from mindspeed_amd.dispatcher import dispatch_mlp_combine
+
+    x, p, idx, w1, w2, _ = make_inputs(cfg, device)
+    with torch.no_grad():
+        for _ in range(warmup):
+            dispatch_mlp_combine(x, idx, p, (w1, w2), fuse_activation=fuse_activation)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            dispatch_mlp_combine(x, idx, p, (w1, w2), fuse_activation=fuse_activation)
+        torch.cuda.synchronize()
+    return round((time.perf_counter() - t0) * 1e3 / steps, 4)
+
+
 def graph_replay_ms(cfg, device, replays=200):
     """One forward+backward step of the layer recorded into a HIP graph (the C ABI only launches kernels on the
     caller's stream, so the step can be captured) and replayed: ms per replay, or None if a replay does not reproduce
@@ -456,6 +474,13 @@ def main():
             torch.cuda.empty_cache()
         others["mixtral_fp32_grad_accumulation"] = acc
 
+    def forward_only_section():
+        others["mixtral_forward_only"] = {
+            "note": "forward pass alone under torch.no_grad(), ms per pass and tokens/s",
+            **{name: {"ms": ms, "tokens_per_s": round(cfg["T"] / (ms / 1e3), 1)}
+               for name, ms in (("one_kernel_per_op", forward_only_ms(cfg, device, False)),
+                                ("fused_activation", forward_only_ms(cfg, device, True)))}}
+
     if not args.no_extras:
         extra("board_mfma_probe", probe_section)
         extra("routing_map_mode", routing_map_section)
@@ -468,6 +493,7 @@ def main():
             if "plumbing" in others:
                 extra("plumbing_graph_replay", graph_section)
             extra("mixtral_fp32_grad_accumulation", accumulation_section)
+            extra("mixtral_forward_only", forward_only_section)
             result["other_workloads"] = others
     if not args.no_cpu_baseline:
         extra("cpu_baseline", lambda: result.__setitem__("cpu_baseline", cpu_baseline(cfg)))

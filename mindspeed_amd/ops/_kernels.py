@@ -369,15 +369,16 @@ _define("gmm_weight_list(Tensor x, Tensor[] weights, Tensor group_list, int grou
 
 
 # ---- grouped matmul with SwiGLU in its epilogue ------------------------------------------------------------------
-def _gmm_swiglu(x, weight, group_list, group_list_type, probs):
+def _gmm_swiglu(x, weight, group_list, group_list_type, probs, want_fc1):
     """``fc1 = grouped_matmul(x, weight)`` and ``act = silu(gate) * up * probs`` from one launch (contiguous 16-bit
-    operands, checked by the Python surface)."""
+    operands, checked by the Python surface).  Without ``want_fc1`` (nothing will be differentiated) the fc1 output is
+    not stored at all and comes back empty."""
     lib = _lib.load()
     dev = x.device
     m, k = x.shape
     ffn = weight.size(2) // 2
     p_code = _lib.dtype_code(probs.dtype, "probs") if probs is not None else 0
-    fc1 = torch.empty((m, 2 * ffn), dtype=x.dtype, device=dev)
+    fc1 = torch.empty((m, 2 * ffn) if want_fc1 else (0,), dtype=x.dtype, device=dev)
     act = torch.empty((m, ffn), dtype=x.dtype, device=dev)
     nbytes = ctypes.c_size_t(0)
     _lib.check(lib.ms_gmm_workspace_size(group_list.numel(), m, 0, ctypes.byref(nbytes)), "ms_gmm_workspace_size")
@@ -385,15 +386,17 @@ def _gmm_swiglu(x, weight, group_list, group_list_type, probs):
     with torch.cuda.device(dev), flop_counter.op("gmm_fwd_swiglu", flop_counter.gmm_flops(m, k, 2 * ffn), "flop", dev):
         _lib.check(lib.ms_gmm_swiglu(
             _lib.stream_ptr(dev), _lib.ptr(x), x.stride(0), x.stride(1), _lib.ptr(weight), weight.stride(0),
-            weight.stride(1), weight.stride(2), _lib.ptr(fc1), 2 * ffn, _lib.ptr(act), ffn, _lib.ptr(probs), p_code,
+            weight.stride(1), weight.stride(2), _lib.ptr(fc1) if want_fc1 else None, 2 * ffn, _lib.ptr(act), ffn,
+            _lib.ptr(probs), p_code,
             _lib.ptr(group_list), group_list_type, group_list.numel(), m, k, ffn, _lib.dtype_code(x.dtype, "x"),
             _lib.ptr(ws), ws.numel()), "ms_gmm_swiglu")
     return fc1, act
 
 
-_define("gmm_swiglu(Tensor x, Tensor weight, Tensor group_list, int group_list_type, Tensor? probs) -> (Tensor, Tensor)",
-        _gmm_swiglu, lambda x, weight, group_list, group_list_type, probs:
-        (x.new_empty((x.size(0), weight.size(2))), x.new_empty((x.size(0), weight.size(2) // 2))))
+_define("gmm_swiglu(Tensor x, Tensor weight, Tensor group_list, int group_list_type, Tensor? probs, bool want_fc1) "
+        "-> (Tensor, Tensor)",
+        _gmm_swiglu, lambda x, weight, group_list, group_list_type, probs, want_fc1:
+        (x.new_empty((x.size(0), weight.size(2)) if want_fc1 else (0,)), x.new_empty((x.size(0), weight.size(2) // 2))))
 
 
 def _gmm_swiglu_grad(dy, w2, fc1, probs, group_list, group_list_type):

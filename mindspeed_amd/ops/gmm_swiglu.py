@@ -7,7 +7,8 @@ recomputation the activation is dropped after the second matmul and rebuilt from
 (:121-127,183-191).  Here the first two are one kernel launch: every tile of the first grouped matmul
 holds 128 gate columns and the matching 128 up columns, and its epilogue writes both the fc1 output (kept
 for backward, exactly as the reference keeps it) and the activation, computed from the already rounded
-fc1 values — bit for bit what the stand-alone SwiGLU kernel produces from the stored fc1 output.
+fc1 values — bit for bit what the stand-alone SwiGLU kernel produces from the stored fc1 output.  Where
+nothing is differentiated (inference, ``torch.no_grad()``) the fc1 output is not written at all.
 
 Backward is the reference's: SwiGLU backward on the saved fc1 output (which also yields the gradient of
 the probabilities), then dX and dW of the grouped matmul.  ``recompute_activation=True`` keeps only the
@@ -25,7 +26,7 @@ from .gmm import _beside, _group_list_tensor, gmm_raw
 __all__ = ["gmm_swiglu", "GmmSwigluFunction", "grouped_mlp", "GroupedMLPFunction"]
 
 
-def _gmm_swiglu_forward(x, weight, group_list, group_list_type, probs):
+def _gmm_swiglu_forward(x, weight, group_list, group_list_type, probs, want_fc1=True):
     _lib.require_device(x, "x")
     _lib.require_device(weight, "weight")
     if x.dim() != 2 or weight.dim() != 3 or weight.size(1) != x.size(1) or weight.size(2) % 2 != 0:
@@ -48,15 +49,18 @@ def _gmm_swiglu_forward(x, weight, group_list, group_list_type, probs):
         if p.numel() != m:
             raise RuntimeError(f"probs has {p.numel()} entries, expected {m}")
         _lib.dtype_code(p.dtype, "probs")
-    fc1, act = K.gmm_swiglu(x, weight, gl, group_list_type, p)
-    return fc1, act, gl, p
+    fc1, act = K.gmm_swiglu(x, weight, gl, group_list_type, p, want_fc1)
+    return (fc1 if want_fc1 else None), act, gl, p
 
 
 class GmmSwigluFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, group_list, group_list_type, probs):
-        fc1, act, gl, p = _gmm_swiglu_forward(x, weight, group_list, group_list_type, probs)
-        ctx.save_for_backward(x, weight, gl, fc1, p)
+        # the fc1 output exists for the backward pass only: where nothing is differentiated (inference) it is not stored
+        differentiated = any(ctx.needs_input_grad)
+        fc1, act, gl, p = _gmm_swiglu_forward(x, weight, group_list, group_list_type, probs, want_fc1=differentiated)
+        if differentiated:
+            ctx.save_for_backward(x, weight, gl, fc1, p)
         ctx.group_list_type = group_list_type
         ctx.probs_shape = None if probs is None else probs.shape
         return act
@@ -120,8 +124,9 @@ class GroupedMLPFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, w1, w2, group_list, group_list_type, probs, recompute_activation, fused_kernels):
+        differentiated = any(ctx.needs_input_grad)
         if fused_kernels:
-            fc1, act, gl, p = _gmm_swiglu_forward(x, w1, group_list, group_list_type, probs)
+            fc1, act, gl, p = _gmm_swiglu_forward(x, w1, group_list, group_list_type, probs, want_fc1=differentiated)
         else:
             _lib.require_device(x, "x")
             gl = _group_list_tensor(group_list, x.device)
@@ -138,7 +143,8 @@ class GroupedMLPFunction(torch.autograd.Function):
         if w2.dim() != 3 or w2.size(0) != w1.size(0) or w2.size(1) != act.size(1) or w2.dtype != x.dtype:
             raise ValueError(f"w2 {tuple(w2.shape)} {w2.dtype} does not match the activation {tuple(act.shape)} {act.dtype}")
         out = gmm_raw(act, w2, gl, 0, group_list_type)
-        ctx.save_for_backward(x, w1, w2, gl, fc1, p, None if recompute_activation else act)
+        if differentiated:
+            ctx.save_for_backward(x, w1, w2, gl, fc1, p, None if recompute_activation else act)
         ctx.group_list_type = group_list_type
         ctx.fused_kernels = fused_kernels
         ctx.probs_shape = None if probs is None else probs.shape

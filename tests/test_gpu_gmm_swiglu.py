@@ -185,3 +185,26 @@ def _grouped_mlp_case(counts, K, ffn, dtype, pdt, extra, recompute, fused_kernel
     assert rel_l2(w1f.grad, w164.grad) <= tol and rel_l2(w2f.grad, w264.grad) <= tol
     if probs is not None:
         assert rel_l2(pf.grad, p64.grad) <= tol
+
+
+def test_inference_skips_the_fc1_output(device):
+    """Under ``torch.no_grad()`` the fused forward does not store the fc1 output (the kernel's NULL-output form):
+    the activation and the MLP output are bit for bit those of the differentiable call."""
+    say("fused forward without fc1 output")
+    counts, K, ffn, dtype = [130, 256, 1, 300, 64, 0, 200, 73], 256, 384, torch.bfloat16
+    M, E = sum(counts) + 5, len(counts)
+    gen = torch.Generator().manual_seed(23)
+    x = torch.randn(M, K, generator=gen).to(dtype).to(device)
+    w1 = (torch.randn(E, K, 2 * ffn, generator=gen) * 0.05).to(dtype).to(device)
+    w2 = (torch.randn(E, ffn, K, generator=gen) * 0.05).to(dtype).to(device)
+    probs = torch.rand(M, generator=gen).to(device)
+    gl = torch.tensor(counts, dtype=torch.int64, device=device)
+    act = ops.gmm_swiglu(x.clone().requires_grad_(True), w1, gl, probs)
+    out = ops.grouped_mlp(x.clone().requires_grad_(True), w1, w2, gl, probs)
+    before = torch.cuda.memory_allocated(device)
+    with torch.no_grad():
+        act_inf = ops.gmm_swiglu(x, w1, gl, probs)
+        assert torch.cuda.memory_allocated(device) - before < 2 * act_inf.numel() * act_inf.element_size() + (1 << 20)
+        out_inf = ops.grouped_mlp(x, w1, w2, gl, probs)
+    torch.cuda.synchronize()
+    assert torch.equal(act_inf, act.detach()) and torch.equal(out_inf, out.detach())

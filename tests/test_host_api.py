@@ -242,6 +242,8 @@ def test_shapes_propagate_on_meta_tensors():
     assert act.shape == (T * K, F) and act.dtype == torch.bfloat16
     act.sum().backward()
     assert xs.grad.shape == xs.shape and rp.grad.shape == rp.shape
+    with torch.no_grad():
+        assert gmm_swiglu(xs, w1, gl, rp).shape == (T * K, F) and grouped_mlp(xs, w1, w2, gl, rp).shape == (T * K, H)
     for fused in (True, False):
         for recompute in (False, True):
             xm = meta(T * K, H, grad=True)
