@@ -208,3 +208,25 @@ def test_inference_skips_the_fc1_output(device):
         out_inf = ops.grouped_mlp(x, w1, w2, gl, probs)
     torch.cuda.synchronize()
     assert torch.equal(act_inf, act.detach()) and torch.equal(out_inf, out.detach())
+
+
+def test_layer_default_under_no_grad_is_the_fused_form(device):
+    """``dispatch_mlp_combine`` without a ``fuse_activation`` argument: one kernel per op where gradients may follow,
+    the fused form under ``torch.no_grad()``; both give the same bits."""
+    say("layer default under no_grad")
+    from mindspeed_amd import flop_counter
+    T, H, E, K, F, dtype = 512, 256, 8, 2, 384, torch.bfloat16
+    gen = torch.Generator().manual_seed(5)
+    x = torch.randn(T, H, generator=gen).to(dtype).to(device)
+    p, idx = O.route_topk(torch.randn(T, E, generator=gen), K)
+    p, idx = p.to(dtype).to(device), idx.to(device)
+    w1 = (torch.randn(E, H, 2 * F, generator=gen) * 0.05).to(dtype).to(device)
+    w2 = (torch.randn(E, F, H, generator=gen) * 0.05).to(dtype).to(device)
+    with flop_counter.record(timing=False) as rec:
+        with_grad = dispatch_mlp_combine(x.clone().requires_grad_(True), idx, p, (w1, w2))
+    assert "swiglu" in rec.summary() and "gmm_fwd_swiglu" not in rec.summary()
+    with torch.no_grad(), flop_counter.record(timing=False) as rec:
+        inference = dispatch_mlp_combine(x, idx, p, (w1, w2))
+        separate = dispatch_mlp_combine(x, idx, p, (w1, w2), fuse_activation=False)
+    assert "gmm_fwd_swiglu" in rec.summary()
+    assert torch.equal(inference, with_grad.detach()) and torch.equal(inference, separate)
