@@ -202,6 +202,13 @@ int ms_gmm_workspace_size_split(int64_t num_groups, int64_t m, int64_t k, int64_
  * column panels, chosen for L2 reuse).  Evaluates the function the kernels call, so a test can check that
  * the order visits every tile exactly once. */
 int ms_gmm_tile_order(int num_row_tiles, int num_col_tiles, int index, int *row_tile, int *col_tile);
+/* Diagnostic, host only (no counterpart in the reference): the number of workgroups per XCD (an eighth of the
+ * grid) that ms_gmm launches for a 16-bit problem of these sizes.  lists: the launch may deal whole groups out to
+ * single XCDs (16 to 256 groups); split: it may split the reduction of its tail tiles.  A test can check with it
+ * that no table the schedule kernel writes needs more slots than the launch has: with per-XCD lists and a split on
+ * the reduction dim (group_type 2) the fullest XCD holds ceil(num_groups / 8) whole output blocks. */
+int ms_gmm_launch_slots(int64_t num_groups, int64_t m, int64_t k, int64_t n, int group_type, int lists,
+                        int split, int64_t *slots_per_xcd);
 int ms_gmm(ms_stream_t stream, const void *x, int64_t x_stride0, int64_t x_stride1,
            const void *weight, int64_t w_stride_group, int64_t w_stride0, int64_t w_stride1,
            void *y, int64_t y_stride_row, const int64_t *group_list, int group_list_type,

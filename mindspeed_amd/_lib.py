@@ -45,6 +45,7 @@ _SIGNATURES = {
     "ms_moe_routing_map_probs_grad": [_c_void_p, _c_void_p, _i64, _c_void_p, _int, _i64, _c_void_p],
     "ms_gmm_workspace_size": [_i64, _i64, _int, ctypes.POINTER(_size_t)],
     "ms_gmm_tile_order": [_int, _int, _int, ctypes.POINTER(_int), ctypes.POINTER(_int)],
+    "ms_gmm_launch_slots": [_i64, _i64, _i64, _i64, _int, _int, _int, ctypes.POINTER(_i64)],
     "ms_gmm_workspace_size_split": [_i64, _i64, _i64, _i64, _int, _int, _int, _int, ctypes.POINTER(_size_t)],
     "ms_gmm": [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _i64, _i64, _i64, _c_void_p, _i64, _c_void_p, _int, _int,
                _i64, _i64, _i64, _i64, _int, _int, _int, _c_void_p, _size_t],

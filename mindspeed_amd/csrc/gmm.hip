@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
                                                            int64_t b_stride_group, int64_t c_stride_group,
                                                            const int64_t *__restrict__ b_offsets, TileTable *table,
                                                            SplitTail *split_records, int split_cols, int split_cus,
-                                                           GroupEntry *members) {
+                                                           GroupEntry *members, int slot_budget) {
     extern __shared__ int64_t ends[];          // [num_groups] clamped end offset of every group
     __shared__ int64_t scratch64[4];
     __shared__ ScanItem scratch_item[4];
@@ -285,6 +285,13 @@ __global__ __launch_bounds__(256) void gmm_schedule_kernel(const int64_t *__rest
                 max_load = xcd_load[q] > max_load ? xcd_load[q] : max_load;
             }
             lists_ok = total > 0 && static_cast<long long>(max_load) * 800 <= total * 103 ? 1 : 0;
+            // never more slots than the launch has workgroups for: the tiles beyond would stay unwritten
+            int most_groups = 0;
+            for (int q = 0; q < 8; ++q) most_groups = xcd_count[q] > most_groups ? xcd_count[q] : most_groups;
+            const long long zero_fill = group_type == 0 && ends[num_groups - 1] < m
+                ? ((static_cast<long long>((m - static_cast<int>(ends[num_groups - 1]) + tile_rows - 1) / tile_rows) * num_col_tiles + 7) >> 3) : 0;
+            const long long need = group_type == 0 ? max_load + zero_fill : static_cast<long long>(most_groups) * out_tiles;
+            if (need > slot_budget) lists_ok = 0;
         }
         __syncthreads();
         lists = lists_ok != 0;
@@ -848,6 +855,30 @@ constexpr size_t workspace_need(int64_t num_groups) {
 // ... and, for launches that may split the reduction of their small tail tiles, the fp32 partial sums behind that
 constexpr size_t split_ws_pos(int64_t num_groups) { return (workspace_need(num_groups) + 255) & ~static_cast<size_t>(255); }
 
+// Slots (workgroups) per XCD that a launch must provide: no table the schedule kernel can write needs more.
+//   common table: every entry rounds its eighth of its tiles up, so an eighth of all tiles plus one slot per entry;
+//   a launch that may split its tail tiles has up to kMaxSplit entries per tail and up to kSplitCus more tiles;
+//   per-XCD lists, split on rows: the fullest XCD holds at most 1.03 times an eighth of all tiles (the schedule kernel's
+//   own balance test) plus its eighth of the zero-fill pseudo-group;
+//   per-XCD lists, split on the reduction dim: every group has the same number of output tiles and the XCD with the
+//   most groups holds ceil(num_groups / 8) of them, however short their reductions are (an empty group still writes
+//   its block of zeros), which exceeds an eighth of all tiles whenever num_groups is not a multiple of 8.
+int64_t launch_slots_per_xcd(int group_type, int64_t num_groups, int64_t m, int64_t k, int64_t tile_rows,
+                             int64_t num_col_tiles, bool lists, bool split) {
+    const int64_t row_tiles_bound = group_type == 0 ? ceil_div(m, tile_rows) + num_groups + 2
+                                                    : num_groups * (k / tile_rows + 1);
+    const int64_t tiles_bound = row_tiles_bound * num_col_tiles;
+    int64_t slots = split ? ceil_div(tiles_bound + kSplitCus, 8) + (1 + kMaxSplit) * num_groups + 2
+                          : ceil_div(tiles_bound, 8) + 2 * num_groups + 2;
+    if (lists) {
+        const int64_t by_lists = group_type == 0
+            ? ceil_div(tiles_bound + tiles_bound / 25, 8) + 2 * num_groups + 2
+            : ceil_div(num_groups, 8) * ceil_div(k, tile_rows) * num_col_tiles;
+        slots = by_lists > slots ? by_lists : slots;
+    }
+    return slots;
+}
+
 // Whether a launch of these sizes can come to split its tail tiles at all (the schedule kernel decides from the
 // group list whether it does), and how many bytes of partial sums it may then write: the parts of a launch number at
 // most kSplitCus tiles, i.e. kSplitCus / column tiles blocks of kSplitRows x n floats.
@@ -931,6 +962,17 @@ extern "C" int ms_gmm_workspace_size(int64_t num_groups, int64_t m, int group_ty
     MS_REQUIRE(num_groups >= 1 && num_groups <= kMaxGroups, MS_ERR_UNSUPPORTED,
                "ms_gmm_workspace_size: num_groups %lld outside [1, %d]", (long long)num_groups, kMaxGroups);
     *bytes = (workspace_need(num_groups) + 255) & ~static_cast<size_t>(255);
+    return MS_OK;
+}
+
+// Workgroups per XCD that ms_gmm launches for a 16-bit problem of these sizes (grid = 8 times that): host arithmetic
+// only.  lists / split: whether the launch may deal whole groups out to single XCDs / split the reduction of its tail tiles.
+extern "C" int ms_gmm_launch_slots(int64_t num_groups, int64_t m, int64_t k, int64_t n, int group_type, int lists,
+                                   int split, int64_t *slots_per_xcd) {
+    MS_REQUIRE(slots_per_xcd != nullptr && num_groups >= 1 && num_groups <= kMaxGroups && m >= 0 && k >= 0 && n >= 0 &&
+                   (group_type == 0 || group_type == 2),
+               MS_ERR_INVALID_ARGUMENT, "ms_gmm_launch_slots: bad arguments");
+    *slots_per_xcd = launch_slots_per_xcd(group_type, num_groups, m, k, BM, ceil_div(n, BN), lists != 0, split != 0);
     return MS_OK;
 }
 
@@ -1071,13 +1113,17 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     GroupEntry *members = num_groups >= 16 && num_groups <= kMaxListGroups &&
                                   (group_type == 0 || (a_stride_row == 1 && b_stride_col == 1 && a_stride_red != 1 && b_stride_red != 1))
         ? reinterpret_cast<GroupEntry *>(static_cast<char *>(workspace) + members_pos(num_groups)) : nullptr;
+    const int64_t slots_per_xcd = launch_slots_per_xcd(group_type, num_groups, m, k, tile_rows, num_col_tiles,
+                                                       members != nullptr, split_ws != nullptr);
+    MS_REQUIRE(slots_per_xcd < (1ll << 27), MS_ERR_UNSUPPORTED, "ms_gmm: problem too large (%lld slots per XCD)",
+               (long long)slots_per_xcd);
     auto schedule = [&](int split_tails) -> int {
         hipLaunchKernelGGL(gmm_schedule_kernel, dim3(1), dim3(256), static_cast<size_t>(num_groups) * sizeof(int64_t),
                            stream, group_list, group_list_type, group_type, static_cast<int>(num_groups),
                            static_cast<int>(m), static_cast<int>(k), tile_rows, static_cast<int>(num_col_tiles),
                            split_tails, kTailsLastRounds * num_cus, w_stride_group, c_stride_group, b_offsets, table,
                            split_tails ? split_records : nullptr, static_cast<int>(n), num_cus,
-                           split_tails ? members : nullptr);
+                           split_tails ? members : nullptr, static_cast<int>(slots_per_xcd));
         MS_CHECK_LAUNCH("gmm_schedule_kernel");
         return MS_OK;
     };
@@ -1094,13 +1140,7 @@ static int gmm_impl(ms_stream_t stream_, const void *x, int64_t x_stride0, int64
     args.c_stride_row = y_stride_row;
     args.cols = static_cast<int>(n);
     args.num_col_tiles = static_cast<int>(num_col_tiles);
-    // slots per XCD: every entry rounds its tiles up to a multiple of 8; a launch that may split its tail tiles has up
-    // to kMaxSplit entries per tail and up to kSplitCus more tiles
-    // (a launch that may deal whole groups out to the XCDs has up to 1.03 times an eighth of all tiles as slots)
-    const int64_t slot_tiles = members != nullptr ? tiles_bound + tiles_bound / 25 : tiles_bound;
-    const unsigned grid = split_ws == nullptr
-        ? static_cast<unsigned>((ceil_div(slot_tiles, 8) + 2 * num_groups + 2) * 8)
-        : static_cast<unsigned>((ceil_div(slot_tiles + kSplitCus, 8) + (1 + kMaxSplit) * num_groups + 2) * 8);
+    const unsigned grid = static_cast<unsigned>(slots_per_xcd * 8);
 
     if (swiglu != nullptr) {
         args.cols = static_cast<int>(n / 2);

@@ -197,8 +197,14 @@ def _add_group_bias(y, bias, group_list, group_list_type):
     num_groups = gl.numel()
     if bias.dim() != 2 or bias.size(0) != num_groups or bias.size(1) != y.size(1):
         raise ValueError(f"bias must be [{num_groups}, {y.size(1)}], got {tuple(bias.shape)}")
-    ends = gl if group_list_type == 0 else torch.cumsum(gl, dim=0)
-    rows = torch.arange(y.size(0), device=y.device)
+    # the group ends exactly as the kernels derive them: a cumulative list never runs backwards and never past the
+    # row count, negative counts read as zero (and the vector handed to searchsorted is then always sorted)
+    m = y.size(0)
+    if group_list_type == 0:
+        ends = torch.cummax(gl, dim=0).values.clamp(0, m)
+    else:
+        ends = gl.clamp(0, m).cumsum(dim=0).clamp(max=m)
+    rows = torch.arange(m, device=y.device)
     group = torch.searchsorted(ends, rows, right=True)
     covered = (group < num_groups).unsqueeze(1)
     picked = bias.index_select(0, group.clamp(max=num_groups - 1)).float()

@@ -55,9 +55,10 @@ def _gmm_swiglu_forward(x, weight, group_list, group_list_type, probs, want_fc1=
 
 class GmmSwigluFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, group_list, group_list_type, probs):
-        # the fc1 output exists for the backward pass only: where nothing is differentiated (inference) it is not stored
-        differentiated = any(ctx.needs_input_grad)
+    def forward(ctx, x, weight, group_list, group_list_type, probs, differentiated=True):
+        # the fc1 output exists for the backward pass only: where nothing is differentiated (inference) it is not
+        # stored.  The caller decides (see _differentiated): ctx.needs_input_grad mirrors the inputs' requires_grad
+        # whatever the grad mode, so it cannot tell torch.no_grad() from training.
         fc1, act, gl, p = _gmm_swiglu_forward(x, weight, group_list, group_list_type, probs, want_fc1=differentiated)
         if differentiated:
             ctx.save_for_backward(x, weight, gl, fc1, p)
@@ -82,7 +83,12 @@ class GmmSwigluFunction(torch.autograd.Function):
         elif ctx.needs_input_grad[0]:
             dx = gmm_raw(d_fc1, weight.transpose(1, 2), gl, 0, glt)
         gp_out = gp.view(ctx.probs_shape) if (gp is not None and ctx.needs_input_grad[4]) else None
-        return dx, dw, None, None, gp_out
+        return dx, dw, None, None, gp_out, None
+
+
+def _differentiated(*tensors) -> bool:
+    """Whether autograd will record the call: grad mode on and some input asks for a gradient."""
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
 
 
 def gmm_swiglu(x, weight, group_list, probs=None, *, group_list_type: int = 1):
@@ -93,7 +99,7 @@ def gmm_swiglu(x, weight, group_list, probs=None, *, group_list_type: int = 1):
     Needs the vector-access layout (16-byte aligned tensors, ``K`` and ``ffn`` multiples of 8); otherwise the
     library reports it and the caller can run ``npu_gmm`` and ``swiglu_with_probs`` one after the other.
     """
-    return GmmSwigluFunction.apply(x, weight, group_list, group_list_type, probs)
+    return GmmSwigluFunction.apply(x, weight, group_list, group_list_type, probs, _differentiated(x, weight, probs))
 
 
 def _swiglu_from_fc1(fc1, p):
@@ -123,8 +129,8 @@ class GroupedMLPFunction(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, x, w1, w2, group_list, group_list_type, probs, recompute_activation, fused_kernels):
-        differentiated = any(ctx.needs_input_grad)
+    def forward(ctx, x, w1, w2, group_list, group_list_type, probs, recompute_activation, fused_kernels,
+                differentiated=True):
         if fused_kernels:
             fc1, act, gl, p = _gmm_swiglu_forward(x, w1, group_list, group_list_type, probs, want_fc1=differentiated)
         else:
@@ -177,7 +183,7 @@ class GroupedMLPFunction(torch.autograd.Function):
         dx = gmm_raw(d_fc1, w1.transpose(1, 2), gl, 0, glt) if ctx.needs_input_grad[0] else None
         side.join()
         gp_out = gp.view(ctx.probs_shape) if (gp is not None and ctx.needs_input_grad[5]) else None
-        return dx, dw1, dw2, None, None, gp_out, None, None
+        return dx, dw1, dw2, None, None, gp_out, None, None, None
 
 
 def grouped_mlp(x, w1, w2, group_list, probs=None, *, group_list_type: int = 1, recompute_activation: bool = False,
@@ -186,4 +192,5 @@ def grouped_mlp(x, w1, w2, group_list, probs=None, *, group_list_type: int = 1, 
     ``w1 [E, K, 2*ffn]``, ``w2 [E, ffn, K']``.  ``fused_kernels`` (default) fuses both SwiGLU passes into the
     neighbouring grouped matmuls and needs the layout conditions of :func:`gmm_swiglu`; without it every op is
     its own kernel, for any dtype and layout the grouped matmul takes."""
-    return GroupedMLPFunction.apply(x, w1, w2, group_list, group_list_type, probs, recompute_activation, fused_kernels)
+    return GroupedMLPFunction.apply(x, w1, w2, group_list, group_list_type, probs, recompute_activation, fused_kernels,
+                                    _differentiated(x, w1, w2, probs))

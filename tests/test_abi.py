@@ -95,3 +95,35 @@ def test_tile_order_visits_every_tile_once():
                     assert len({r for r, _ in chunk}) == 4 and len({c for _, c in chunk}) == 8, (R, C, b)
     assert lib.ms_gmm_tile_order(4, 4, 16, ctypes.byref(row), ctypes.byref(col)) != 0
     assert lib.ms_gmm_tile_order(0, 4, 0, ctypes.byref(row), ctypes.byref(col)) != 0
+
+
+def test_launch_has_slots_for_every_table_the_schedule_can_write():
+    """Workgroups per XCD of a grouped-matmul launch against the most slots a tile table can need (host arithmetic).
+    Common table: every group's eighth of its tiles, rounded up.  Per-XCD lists with the split on the reduction dim:
+    the XCD with the most groups holds ceil(G / 8) output blocks, e.g. 3 of 17, which is more than an eighth of all
+    tiles when G is not a multiple of 8."""
+    lib = _lib.load()
+    slots = ctypes.c_int64(0)
+    cdiv = lambda a, b: -(-a // b)
+    for G in (1, 8, 16, 17, 20, 23, 24, 31, 33, 64, 100, 255, 256):
+        for k, n in ((2048, 8192), (2880, 2880), (256, 256), (4096, 4096), (8, 8), (1000, 520)):
+            out_tiles = cdiv(k, 256) * cdiv(n, 256)
+            for lists in (0, 1):
+                assert lib.ms_gmm_launch_slots(G, 4096, k, n, 2, lists, 0, ctypes.byref(slots)) == 0
+                need_common = G * cdiv(out_tiles, 8)
+                assert slots.value >= need_common, (G, k, n, lists, slots.value, need_common)
+                if lists:
+                    need_lists = cdiv(G, 8) * out_tiles
+                    assert slots.value >= need_lists, (G, k, n, slots.value, need_lists)
+    # split on rows: at most ceil(m / 256) + G + 1 row tiles (every group and the zero-fill pseudo-group may end in a
+    # partly filled one); with lists the fullest XCD holds at most 1.03 times an eighth of the groups' tiles plus its
+    # eighth of the pseudo-group's, rounded up
+    for G in (8, 17, 64, 256):
+        for m, n in ((8192, 4096), (65536, 2816), (100, 8)):
+            tiles = (cdiv(m, 256) + G + 1) * cdiv(n, 256)
+            assert lib.ms_gmm_launch_slots(G, m, 4096, n, 0, 1, 0, ctypes.byref(slots)) == 0
+            assert slots.value >= cdiv(tiles * 103, 800) + 1
+            assert lib.ms_gmm_launch_slots(G, m, 4096, n, 0, 0, 1, ctypes.byref(slots)) == 0
+            assert slots.value >= cdiv(tiles + 256, 8) + G
+    assert lib.ms_gmm_launch_slots(0, 1, 1, 1, 0, 0, 0, ctypes.byref(slots)) != 0
+    assert lib.ms_gmm_launch_slots(8, 1, 1, 1, 1, 0, 0, ctypes.byref(slots)) != 0

@@ -136,6 +136,47 @@ def test_forward_and_backward_vs_oracle(M, K, N, E, kind, dtype, device):
     assert torch.equal(y2, y.detach())
 
 
+@pytest.mark.parametrize("E,empty,K,N,rows", [
+    (17, (16,), 2048, 4096, 256),          # 16 groups of 256 rows and one empty: the XCD with three groups has 3 x 128 tiles
+    (20, (3, 8, 13, 19), 2880, 2880, 192),  # 16 + 4 empty, 12 x 12 output tiles per group
+    (23, (), 1024, 2048, 128),             # no empty group; 23 groups deal out as 3, 3, 3, 3, 3, 3, 3, 2
+])
+def test_weight_gradient_group_count_not_a_multiple_of_8(E, empty, K, N, rows, device):
+    """Split on the reduction dim with whole groups dealt out to single XCDs: the XCD with the most groups holds
+    ceil(E / 8) whole output blocks, more than an eighth of all tiles when E is not a multiple of 8 (with empty groups
+    ranked last the reduction lengths still balance, so the lists are taken).  Every tile of every block must be
+    written, and an empty group's block must be exactly zero (test_npu_gmm.py:105-113 in the reference).  The output
+    buffer is poisoned first through the caching allocator."""
+    say("dW lists", E, empty, K, N, rows)
+    counts = torch.tensor([0 if g in empty else rows for g in range(E)])
+    M = int(counts.sum())
+    gen = torch.Generator().manual_seed(E)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    gy = torch.randn(M, N, generator=gen).to(torch.bfloat16)
+    exp = O.gmm(x.t(), gy, counts, 2, 1)
+    xd, gyd, gl = x.to(device), gy.to(device), counts.to(device)
+    for form in ("counts", "cumulative"):
+        poison = torch.full((E, K, N), float("nan"), dtype=torch.bfloat16, device=device)
+        del poison
+        if form == "counts":
+            got = ops.npu_gmm_v2(xd.t(), gyd, group_list=gl, group_type=2)
+        else:
+            got = ops.npu_gmm(xd.t(), gyd, group_list=torch.cumsum(counts, 0).tolist(), group_type=2)
+        torch.cuda.synchronize()
+        assert got.shape == (E, K, N)
+        assert not torch.isnan(got).any(), "tiles of the weight gradient were left unwritten"
+        assert rel_l2(got, exp) <= 1e-2
+        for g in empty:
+            assert torch.count_nonzero(got[g]) == 0
+    # the fp32 `+=` form (npu_groupmatmul_add_fp32) on the same launch shape
+    acc = torch.ones(E * K, N, dtype=torch.float32, device=device)
+    ops.npu_groupmatmul_add_fp32(xd, gyd, torch.cumsum(counts, 0).to(device), acc)
+    torch.cuda.synchronize()
+    assert rel_l2(acc.view(E, K, N) - 1.0, exp.float()) <= 1e-2
+    for g in empty:
+        assert torch.equal(acc.view(E, K, N)[g], torch.ones(K, N, device=device))
+
+
 def test_transposed_weight_view_and_raw_module(device):
     """A weight stored [E, N, K] and passed as .transpose(1, 2) (Ops.gmm's trans_b form) needs no copy."""
     gen = torch.Generator().manual_seed(5)

@@ -208,6 +208,25 @@ def test_inference_skips_the_fc1_output(device):
         out_inf = ops.grouped_mlp(x, w1, w2, gl, probs)
     torch.cuda.synchronize()
     assert torch.equal(act_inf, act.detach()) and torch.equal(out_inf, out.detach())
+    # real parameters (requires_grad) under no_grad: still the inference form.  (Inside the autograd function the
+    # inputs' requires_grad is visible whatever the grad mode, so the decision is taken before it.)
+    w1p, w2p = torch.nn.Parameter(w1), torch.nn.Parameter(w2)
+    fc1_bytes = M * 2 * ffn * x.element_size()
+    torch.cuda.reset_peak_memory_stats(device)
+    before = torch.cuda.memory_allocated(device)
+    with torch.no_grad():
+        act_p = ops.gmm_swiglu(x, w1p, gl, probs)
+        out_p = ops.grouped_mlp(x, w1p, w2p, gl, probs)
+    torch.cuda.synchronize()
+    # peak = activation + output + tile table (1.3 MB here); with the fc1 output (1.6 MB) beside the activation it
+    # would be at least 2.4 MB
+    assert torch.cuda.max_memory_allocated(device) - before < fc1_bytes + (1 << 18)
+    assert not act_p.requires_grad and not out_p.requires_grad
+    assert torch.equal(act_p, act.detach()) and torch.equal(out_p, out.detach())
+    # and with grad mode on the same parameters get their gradients
+    out_t = ops.grouped_mlp(x, w1p, w2p, gl, probs)
+    out_t.sum().backward()
+    assert w1p.grad is not None and w2p.grad is not None and torch.equal(out_t.detach(), out.detach())
 
 
 def test_layer_default_under_no_grad_is_the_fused_form(device):
