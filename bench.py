@@ -63,30 +63,6 @@ def measured_traffic(workload, kernel):
     return data.get("bytes_per_launch", {}).get(workload, {}).get(kernel)
 
 
-def board_mfma_rate(seconds=2.0):
-    """What the matrix cores of this board reach by themselves on random bf16 operands: the stand-alone probe
-    `mindspeed_amd/probes/bin/mfma_power` (built by `__graft_entry__.build()`), a loop of v_mfma_f32_32x32x16_bf16
-    with no memory traffic on every CU, run for `seconds` as a child process.  The board's power limit holds the shader
-    clock below the 2.4 GHz that the published peak is quoted at, by an amount that depends on the operand values; this
-    is the rate that limit leaves to a kernel that does nothing but multiply.  None if the probe is not built."""
-    import re
-    import subprocess
-
-    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "mindspeed_amd", "probes", "bin", "mfma_power")
-    if not os.path.exists(exe):
-        return None
-    try:
-        res = subprocess.run([exe, "quick", str(seconds)], capture_output=True, text=True, timeout=60)
-    except (OSError, subprocess.TimeoutExpired):
-        return None
-    m = re.search(r"32x32x16 random: ([\d.]+) TFLOP/s\s+(-?[\d.]+) W\s+(-?[\d.]+) MHz", res.stdout)
-    if res.returncode != 0 or m is None:
-        return None
-    return {"tflops": float(m.group(1)), "board_watts": float(m.group(2)), "shader_mhz": float(m.group(3)),
-            "what": "v_mfma_f32_32x32x16_bf16 back to back on all CUs, random operands in registers, no memory "
-                    f"traffic, {seconds:g} s (mindspeed_amd/probes/mfma_power.hip)"}
-
-
 def _cpu_layer_once(cfg, sample, dtype=torch.float32):
     from oracle import moe_oracle as O
 
@@ -399,13 +375,12 @@ def main():
                         f"bracket reads {empty_bracket_ms * 1e3:.1f} us on this box",
     }
     if args.copy_calibration:
-        from mindspeed_amd import _lib
-        lib = _lib.load()
+        from mindspeed_amd import microbench_kernels
         n = args.copy_calibration << 20
         src = torch.empty(n, dtype=torch.uint8, device=device).fill_(1)
         dst = torch.empty_like(src)
         for _ in range(3):
-            _lib.check(lib.ms_copy_bytes(_lib.stream_ptr(device), _lib.ptr(src), _lib.ptr(dst), n), "ms_copy_bytes")
+            microbench_kernels.copy_bytes(src, dst)
         torch.cuda.synchronize()
         result["copy_calibration_bytes"] = n
     def extra(name, fn):
@@ -418,12 +393,6 @@ def main():
             traceback.print_exc(file=sys.stderr)
             result.setdefault("extras_failed", {})[name] = repr(exc)
         torch.cuda.empty_cache()
-
-    def probe_section():
-        probe = board_mfma_rate()
-        if probe is not None:
-            result["board_mfma_probe"] = probe
-            roofline["frac_of_board_mfma_probe"] = round(dom["tflops"] / probe["tflops"], 4)
 
     def routing_map_section():
         result["routing_map_mode"] = measure_routing_map_mode(cfg, device, x.detach(), idx, p.detach())
@@ -482,7 +451,6 @@ def main():
                                 ("fused_activation", forward_only_ms(cfg, device, True)))}}
 
     if not args.no_extras:
-        extra("board_mfma_probe", probe_section)
         extra("routing_map_mode", routing_map_section)
         extra("permute_family", permute_family_section)
         if args.workload == "mixtral":

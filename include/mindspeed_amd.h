@@ -159,6 +159,13 @@ int ms_moe_routing_map_probs(ms_stream_t stream, const int32_t *sorted_flat, int
 int ms_moe_routing_map_probs_grad(ms_stream_t stream, const int32_t *row_id_map, int64_t num_entries,
                                   const void *grad_permuted_probs, int dtype, int64_t num_out_tokens,
                                   void *grad_probs);
+/* Rows of a [num_out_tokens, hidden] matrix in permuted layout that no map entry leads to (sorted_flat[r] < 0:
+ * only when num_out_tokens exceeds the number of set entries) are written as zeros, all others left alone.
+ * The gradient of the routing-map unpermute w.r.t. the permuted rows (torch_npu.npu_moe_token_unpermute_with_
+ * routing_map_grad behind mindspeed/te/pytorch/permutation.py:107-148) is completed with it, so that no row of it
+ * is left unwritten. */
+int ms_moe_zero_unmapped_rows(ms_stream_t stream, const int32_t *sorted_flat, int64_t num_out_tokens,
+                              int64_t hidden, int dtype, void *rows);
 
 /* ------------------------------------------------------------------------
  * Grouped matmul — stands in for aclnnGroupedMatmulV2 / V4 as called from
@@ -314,10 +321,12 @@ int ms_sort_chunks(ms_stream_t stream, const void *input, const int64_t *split_s
 int ms_gather_rows(ms_stream_t stream, const void *input, const int32_t *row_map, int64_t rows,
                    int64_t hidden, int dtype, int inverse, void *out);
 
-/* Plain device copy kernel (16-byte vectors, grid-stride).  Used to calibrate
- * profiler byte counters against a transfer of known size. */
-int ms_copy_bytes(ms_stream_t stream, const void *src, void *dst, size_t bytes);
-
+/* The chunk sort's row map alone, in the direction make_chunk_sort_map of the fused form returns it
+ * (mindspeed/lite/ops/triton/sort_chunks_by_idx.py:67-115): row_id_map int32 [rows], entry r = output row of
+ * source row r (-1 for rows past the sum of the sizes).  ms_gather_rows moves rows by it: inverse != 0 is the
+ * forward direction of sort_chunks_by_map (:167-221), inverse == 0 its backward. */
+int ms_chunk_sort_map(ms_stream_t stream, const int64_t *split_sizes, const int64_t *sorted_idxs,
+                      int64_t num_chunks, int64_t rows, int32_t *row_id_map);
 #ifdef __cplusplus
 }
 #endif

@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # MINDSPEED_AMD_LIB names another build of the same library (to compare two builds on one machine)
 LIB_PATH = os.environ.get("MINDSPEED_AMD_LIB") or os.path.join(_HERE, "libmindspeed_amd.so")
 
-ABI_VERSION = 102                # what ms_version() of a matching build returns (argument lists below)
+ABI_VERSION = 103                # what ms_version() of a matching build returns (argument lists below)
 MS_BF16, MS_FP16, MS_FP32 = 0, 1, 2
 MS_INT32, MS_INT64 = 0, 1
 MS_MAX_EXPERTS = 1024
@@ -43,6 +43,7 @@ _SIGNATURES = {
                                    _c_void_p, _c_void_p, _c_void_p, _c_void_p, _size_t],
     "ms_moe_routing_map_probs": [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _int, _c_void_p, _c_void_p],
     "ms_moe_routing_map_probs_grad": [_c_void_p, _c_void_p, _i64, _c_void_p, _int, _i64, _c_void_p],
+    "ms_moe_zero_unmapped_rows": [_c_void_p, _c_void_p, _i64, _i64, _int, _c_void_p],
     "ms_gmm_workspace_size": [_i64, _i64, _int, ctypes.POINTER(_size_t)],
     "ms_gmm_tile_order": [_int, _int, _int, ctypes.POINTER(_int), ctypes.POINTER(_int)],
     "ms_gmm_launch_slots": [_i64, _i64, _i64, _i64, _int, _int, _int, ctypes.POINTER(_i64)],
@@ -63,7 +64,7 @@ _SIGNATURES = {
     "ms_sort_chunks": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _i64, _i64, _i64, _int, _c_void_p, _int,
                        _c_void_p, _c_void_p, _c_void_p],
     "ms_gather_rows": [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _int, _int, _c_void_p],
-    "ms_copy_bytes": [_c_void_p, _c_void_p, _c_void_p, _size_t],
+    "ms_chunk_sort_map": [_c_void_p, _c_void_p, _c_void_p, _i64, _i64, _c_void_p],
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES) + ("ms_last_error",)
 

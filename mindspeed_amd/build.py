@@ -17,6 +17,8 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libmindspeed_amd.so")
 TRACE_LIB_PATH = os.path.join(HERE, "libmindspeed_amd_trace.so")   # diagnostic variant: per-tile time stamps
+MICROBENCH_CSRC = os.path.join(HERE, "csrc_microbench")
+MICROBENCH_LIB_PATH = os.path.join(HERE, "libmindspeed_amd_microbench.so")   # measurement helpers (plain copy kernel)
 
 ARCH = "gfx950"
 # packed-fp32 VALU forms are switched off for every device translation unit.
@@ -97,8 +99,23 @@ def build_trace(verbose: bool = False) -> str:
     return TRACE_LIB_PATH
 
 
+def build_microbench(verbose: bool = False) -> str:
+    """The measurement helpers (csrc_microbench/*.hip: the plain copy kernel the microbenchmarks and the counter
+    calibration use).  A library of its own: nothing in it is part of the product's C ABI."""
+    srcs = sorted(os.path.join(MICROBENCH_CSRC, f) for f in os.listdir(MICROBENCH_CSRC) if f.endswith(".hip"))
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-shared", "-o", MICROBENCH_LIB_PATH, *srcs]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed for the microbench helpers:\n{res.stderr}")
+    if verbose:
+        print(f"built {MICROBENCH_LIB_PATH}")
+    return MICROBENCH_LIB_PATH
+
+
 if __name__ == "__main__":
     if "--trace" in sys.argv:
         build_trace(verbose=True)
+    elif "--microbench" in sys.argv:
+        build_microbench(verbose=True)
     else:
         build(force="--incremental" not in sys.argv, verbose=True)

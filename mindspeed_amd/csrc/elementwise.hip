@@ -219,6 +219,69 @@ __global__ __launch_bounds__(1024) void sort_chunks_kernel(
     }
 }
 
+// The chunk sort's row map by itself, in the direction the reference's make_chunk_sort_map returns it
+// (mindspeed/lite/ops/triton/sort_chunks_by_idx.py:67-115): map[source row] = output row.  Every workgroup scans the
+// chunk sizes in input order (first source row of every chunk) and in output order (first output row of every position),
+// inverts sorted_idxs in LDS, and locates each of its source rows by bisection.  Rows past the sum of the sizes, and
+// rows of chunks that sorted_idxs never names, get -1.
+__global__ __launch_bounds__(256) void chunk_sort_map_kernel(const int64_t *__restrict__ split_sizes,
+                                                             const int64_t *__restrict__ sorted_idxs, int num_chunks,
+                                                             int rows, int32_t *__restrict__ map) {
+    extern __shared__ int lds[];   // src_start[num_chunks + 1], dst_start[num_chunks], pos_of[num_chunks], scratch[32]
+    int *src_start = lds;
+    int *dst_start = lds + num_chunks + 1;
+    int *pos_of = dst_start + num_chunks;
+    int *scratch = pos_of + num_chunks;
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    for (int i = tid; i < num_chunks; i += nthreads) pos_of[i] = -1;
+    __syncthreads();
+    int carry_s = 0, carry_d = 0;
+    for (int c0 = 0; c0 < num_chunks; c0 += nthreads) {
+        const int i = c0 + tid;
+        int size = 0, moved = 0;
+        if (i < num_chunks) {
+            const int64_t sz = split_sizes[i];
+            size = static_cast<int>(sz < 0 ? 0 : (sz > rows ? rows : sz));
+            const int64_t sidx = sorted_idxs[i];
+            if (sidx >= 0 && sidx < num_chunks) {
+                const int64_t ms = split_sizes[sidx];
+                moved = static_cast<int>(ms < 0 ? 0 : (ms > rows ? rows : ms));
+                pos_of[sidx] = i;
+            }
+        }
+        const int s_ex = carry_s + block_exclusive_scan(size, scratch);
+        const int d_ex = carry_d + block_exclusive_scan(moved, scratch);
+        if (i < num_chunks) {
+            src_start[i] = s_ex;
+            dst_start[i] = d_ex;
+        }
+        if (tid == nthreads - 1) {
+            scratch[16] = s_ex + size;
+            scratch[17] = d_ex + moved;
+        }
+        __syncthreads();
+        carry_s = scratch[16];
+        carry_d = scratch[17];
+        __syncthreads();
+    }
+    if (tid == 0) src_start[num_chunks] = carry_s;
+    __syncthreads();
+    const int r = blockIdx.x * nthreads + tid;
+    if (r >= rows) return;
+    int lo = 0, hi = num_chunks + 1;            // last chunk with src_start <= r
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (src_start[mid] <= r) lo = mid; else hi = mid;
+    }
+    int m = -1;
+    if (lo < num_chunks && r < src_start[num_chunks] && pos_of[lo] >= 0) {
+        m = dst_start[pos_of[lo]] + (r - src_start[lo]);
+        if (static_cast<unsigned>(m) >= static_cast<unsigned>(rows)) m = -1;
+    }
+    map[r] = m;
+}
+
 // out[r] = in[row_map[r]] (inverse: out[row_map[r]] = in[r]); `lanes` threads per row, eight 16-byte loads in
 // flight per thread.  Map entries outside [0, rows) move nothing.
 template <typename VecT>
@@ -381,6 +444,21 @@ extern "C" int ms_gather_rows(ms_stream_t stream_, const void *input, const int3
     if (rows == 0) return MS_OK;
     MS_REQUIRE(input && row_map && out, MS_ERR_INVALID_ARGUMENT, "ms_gather_rows: NULL tensor pointer");
     return gather_rows_any(stream, input, out, row_map, rows, hidden, dtype, inverse);
+}
+
+extern "C" int ms_chunk_sort_map(ms_stream_t stream_, const int64_t *split_sizes, const int64_t *sorted_idxs,
+                                 int64_t num_chunks, int64_t rows, int32_t *row_id_map) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MS_REQUIRE(rows >= 0 && rows < (1ll << 31), MS_ERR_INVALID_ARGUMENT, "ms_chunk_sort_map: bad sizes");
+    MS_REQUIRE(num_chunks >= 1 && num_chunks <= 4096, MS_ERR_UNSUPPORTED,
+               "ms_chunk_sort_map: num_chunks %lld outside [1, 4096]", (long long)num_chunks);
+    if (rows == 0) return MS_OK;
+    MS_REQUIRE(split_sizes && sorted_idxs && row_id_map, MS_ERR_INVALID_ARGUMENT, "ms_chunk_sort_map: NULL tensor pointer");
+    const size_t lds = (3 * static_cast<size_t>(num_chunks) + 1 + 32) * sizeof(int);
+    hipLaunchKernelGGL(chunk_sort_map_kernel, dim3(static_cast<unsigned>(ceil_div(rows, 256))), dim3(256), lds, stream,
+                       split_sizes, sorted_idxs, static_cast<int>(num_chunks), static_cast<int>(rows), row_id_map);
+    MS_CHECK_LAUNCH("chunk_sort_map_kernel");
+    return MS_OK;
 }
 
 extern "C" int ms_sort_chunks(ms_stream_t stream_, const void *input, const int64_t *split_sizes,

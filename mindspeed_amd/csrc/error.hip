@@ -34,4 +34,4 @@ hipError_t set_max_dynamic_lds(const void *fn, int bytes) {
 }  // namespace ms
 
 extern "C" const char *ms_last_error(void) { return ms::g_error; }
-extern "C" int ms_version(void) { return 102; }
+extern "C" int ms_version(void) { return 103; }

@@ -630,17 +630,6 @@ __global__ __launch_bounds__(256) void unpermute_grad_kernel(
     }
 }
 
-__global__ __launch_bounds__(256) void copy_bytes_kernel(const v16 *__restrict__ src, v16 *__restrict__ dst,
-                                                         size_t nvec) {
-    for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < nvec;
-         i += static_cast<size_t>(gridDim.x) * blockDim.x)
-        dst[i] = src[i];
-}
-__global__ void copy_tail_kernel(const unsigned char *src, unsigned char *dst, size_t begin, size_t end) {
-    const size_t i = begin + blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
-    if (i < end) dst[i] = src[i];
-}
-
 // ---- pieces shared by the one-launch permute kernels ---------------------------------------
 // The first eight vectors of a thread's source row, as unconditional loads from clamped positions: straight-line
 // code, so that the compiler's waits for loads issued before these can leave them in flight.
@@ -1958,24 +1947,29 @@ extern "C" int ms_moe_routing_map_probs_grad(ms_stream_t stream_, const int32_t 
     return MS_OK;
 }
 
-extern "C" int ms_copy_bytes(ms_stream_t stream_, const void *src, void *dst, size_t bytes) {
+// Rows of a permuted-layout matrix that no map entry leads to (marked by a negative entry of sorted_flat) are written
+// as zeros; all other rows are left alone.
+extern "C" int ms_moe_zero_unmapped_rows(ms_stream_t stream_, const int32_t *sorted_flat, int64_t num_rows, int64_t hidden,
+                                         int dtype, void *rows) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (bytes == 0) return MS_OK;
-    MS_REQUIRE(src && dst, MS_ERR_INVALID_ARGUMENT, "ms_copy_bytes: NULL pointer");
-    size_t nvec = (aligned16(src) && aligned16(dst)) ? bytes / 16 : 0;
-    if (nvec) {
-        size_t blocks = (nvec + 255) / 256;
-        if (blocks > 256 * 32) blocks = 256 * 32;
-        hipLaunchKernelGGL(copy_bytes_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
-                           static_cast<const v16 *>(src), static_cast<v16 *>(dst), nvec);
-        MS_CHECK_LAUNCH("copy_bytes_kernel");
-    }
-    const size_t done = nvec * 16;
-    if (done < bytes) {
-        const size_t rest = bytes - done;
-        hipLaunchKernelGGL(copy_tail_kernel, dim3(static_cast<unsigned>((rest + 255) / 256)), dim3(256), 0, stream,
-                           static_cast<const unsigned char *>(src), static_cast<unsigned char *>(dst), done, bytes);
-        MS_CHECK_LAUNCH("copy_tail_kernel");
-    }
+    const char *fn = "ms_moe_zero_unmapped_rows";
+    MS_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31) && hidden >= 1 && hidden < (1ll << 31), MS_ERR_INVALID_ARGUMENT,
+               "%s: bad sizes", fn);
+    MS_REQUIRE(dtype == MS_BF16 || dtype == MS_FP16 || dtype == MS_FP32, MS_ERR_UNSUPPORTED,
+               "%s: dtype %d is not one of bf16/fp16/fp32", fn, dtype);
+    if (num_rows == 0) return MS_OK;
+    MS_REQUIRE(sorted_flat && rows, MS_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", fn);
+    const int64_t row_bytes = hidden * dtype_size(dtype);
+    const dim3 zgrid(static_cast<unsigned>(ceil_div(num_rows, 4)));
+    if (row_bytes % 16 == 0 && aligned16(rows))
+        hipLaunchKernelGGL(zero_marked_rows_kernel<v16>, zgrid, dim3(256), 0, stream, sorted_flat, static_cast<int>(num_rows),
+                           static_cast<int>(row_bytes / 16), static_cast<v16 *>(rows));
+    else if (dtype == MS_FP32)
+        hipLaunchKernelGGL(zero_marked_rows_kernel<uint32_t>, zgrid, dim3(256), 0, stream, sorted_flat,
+                           static_cast<int>(num_rows), static_cast<int>(row_bytes / 4), static_cast<uint32_t *>(rows));
+    else
+        hipLaunchKernelGGL(zero_marked_rows_kernel<uint16_t>, zgrid, dim3(256), 0, stream, sorted_flat,
+                           static_cast<int>(num_rows), static_cast<int>(row_bytes / 2), static_cast<uint16_t *>(rows));
+    MS_CHECK_LAUNCH("zero_marked_rows_kernel");
     return MS_OK;
 }

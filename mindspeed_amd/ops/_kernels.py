@@ -475,4 +475,50 @@ _define("gather_rows(Tensor src, Tensor row_map, bool zero_fill) -> Tensor", _ga
         lambda src, row_map, zero_fill: torch.empty_like(src))
 
 
+def _chunk_sort_map(split_sizes, sorted_idxs, rows):
+    """int32 ``[rows]``: entry ``r`` = output row of source row ``r`` under the chunk sort (-1 past the chunks)."""
+    lib = _lib.load()
+    dev = split_sizes.device
+    row_id_map = torch.empty(rows, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.ms_chunk_sort_map(_lib.stream_ptr(dev), _lib.ptr(split_sizes), _lib.ptr(sorted_idxs),
+                                         split_sizes.numel(), rows, _lib.ptr(row_id_map)), "ms_chunk_sort_map")
+    return row_id_map
+
+
+_define("chunk_sort_map(Tensor split_sizes, Tensor sorted_idxs, int rows) -> Tensor", _chunk_sort_map,
+        lambda split_sizes, sorted_idxs, rows: split_sizes.new_empty((rows,), dtype=torch.int32))
+
+
+def _move_rows(src, row_map, inverse, zero_fill):
+    """``out[i] = src[row_map[i]]``, or with ``inverse`` ``out[row_map[i]] = src[i]``; rows or vector entries."""
+    lib = _lib.load()
+    dev = src.device
+    out = torch.zeros_like(src) if zero_fill else torch.empty_like(src)
+    rows = src.size(0)
+    width = src.size(1) if src.dim() == 2 else 1
+    with torch.cuda.device(dev):
+        _lib.check(lib.ms_gather_rows(_lib.stream_ptr(dev), _lib.ptr(src), _lib.ptr(row_map), rows, width,
+                                      _lib.dtype_code(src.dtype, "input"), 1 if inverse else 0, _lib.ptr(out)),
+                   "ms_gather_rows")
+    return out
+
+
+_define("move_rows(Tensor src, Tensor row_map, bool inverse, bool zero_fill) -> Tensor", _move_rows,
+        lambda src, row_map, inverse, zero_fill: torch.empty_like(src))
+
+
+def _zero_unmapped_rows(rows, sorted_flat):
+    """Rows ``r`` of ``rows`` with ``sorted_flat[r] < 0`` become zeros, in place."""
+    lib = _lib.load()
+    dev = rows.device
+    with torch.cuda.device(dev):
+        _lib.check(lib.ms_moe_zero_unmapped_rows(_lib.stream_ptr(dev), _lib.ptr(sorted_flat), rows.size(0), rows.size(1),
+                                                 _lib.dtype_code(rows.dtype, "rows"), _lib.ptr(rows)),
+                   "ms_moe_zero_unmapped_rows")
+
+
+_define("zero_unmapped_rows(Tensor(a!) rows, Tensor sorted_flat) -> ()", _zero_unmapped_rows, lambda rows, sorted_flat: None)
+
+
 K = torch.ops.mindspeed_amd

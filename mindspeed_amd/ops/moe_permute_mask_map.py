@@ -28,6 +28,9 @@ from __future__ import annotations
 
 from typing import Optional, Tuple
 
+import os
+import weakref
+
 import torch
 
 from .. import _lib
@@ -76,32 +79,52 @@ def routing_map_row_maps(routing_map: torch.Tensor, num_rows: int, drop_and_pad:
     return (permuted if tokens is not None else None), row_id_map, sorted_flat, (counts if want_counts else None)
 
 
-# The dispatcher hands ``unpermute`` the same ``routing_map`` tensor it gave ``permute``.  The row map that
-# ``permute`` computed from that mask is remembered on the mask tensor itself, so ``unpermute`` need not sort the mask
-# again whatever happened to ``sorted_indices`` in between (clones, views, an exchange between ranks).  It is only used
-# while the mask is that same tensor object in the same state (version counter) and the row count and mode match;
-# any other mask, a view or a copy of it included, is sorted afresh.
+# The dispatcher hands ``unpermute`` the same ``routing_map`` tensor it gave ``permute``.  The row maps that
+# ``permute`` computed from that mask are remembered on the mask tensor itself, so ``unpermute`` need not sort the mask
+# again whatever happened to ``sorted_indices`` in between (clones, views, an exchange between ranks).  They are only
+# used while the mask is that same tensor object in the same state — version counter, storage address and shape — and
+# the row count and mode match; any other mask, a view or a copy of it included, is sorted afresh.  A write that
+# bypasses the version counter (``routing_map.data.copy_()``, ``set_()`` onto the same address, a write through a
+# DLPack / numpy alias) is not seen: a mask changed that way must be permuted again before it is unpermuted, or the
+# memory switched off with ``MINDSPEED_AMD_ROW_MAP_CACHE=0``.  A map reused on another stream than the one that
+# produced it first waits for that stream.
 _ROW_MAPS_KEPT = 4
+_ROW_MAP_CACHE = os.environ.get("MINDSPEED_AMD_ROW_MAP_CACHE", "1") != "0"
+_CHECK_SORTED_INDICES = os.environ.get("MINDSPEED_AMD_CHECK_SORTED_INDICES", "1") != "0"
 
 
-def _remember_row_map(routing_map, num_rows, drop_and_pad, row_id_map):
-    if _tracing(routing_map):
+def _mask_state(routing_map):
+    return (routing_map._version, routing_map.data_ptr(), tuple(routing_map.shape), tuple(routing_map.stride()))
+
+
+def _remember_row_map(routing_map, num_rows, drop_and_pad, row_id_map, sorted_flat, sorted_indices=None):
+    if not _ROW_MAP_CACHE or _tracing(routing_map):
         return
     kept = getattr(routing_map, "_ms_row_maps", None)
-    if kept is None or kept[0] != routing_map._version:
-        kept = (routing_map._version, {})
+    state = _mask_state(routing_map)
+    if kept is None or kept[0] != state:
+        kept = (state, {})
         routing_map._ms_row_maps = kept
     maps = kept[1]
-    maps[(int(num_rows), bool(drop_and_pad))] = row_id_map
+    maps[(int(num_rows), bool(drop_and_pad))] = (row_id_map, sorted_flat, torch.cuda.current_stream(routing_map.device),
+                                                 None if sorted_indices is None else weakref.ref(sorted_indices))
     while len(maps) > _ROW_MAPS_KEPT:
         maps.pop(next(iter(maps)))
 
 
 def _recall_row_map(routing_map, num_rows, drop_and_pad):
+    """``(row_id_map, sorted_flat, sorted_indices or None)`` of an earlier ``permute`` of this very mask, or None."""
     kept = getattr(routing_map, "_ms_row_maps", None)
-    if kept is None or kept[0] != routing_map._version:
+    if not _ROW_MAP_CACHE or kept is None or kept[0] != _mask_state(routing_map):
         return None
-    return kept[1].get((int(num_rows), bool(drop_and_pad)))
+    hit = kept[1].get((int(num_rows), bool(drop_and_pad)))
+    if hit is None:
+        return None
+    row_id_map, sorted_flat, stream, own = hit
+    now = torch.cuda.current_stream(routing_map.device)
+    if now != stream:
+        now.wait_stream(stream)          # everything queued on the producing stream so far, the map's kernel included
+    return row_id_map, sorted_flat, (own() if own is not None else None)
 
 
 def _tracing(t):
@@ -154,7 +177,7 @@ class MoePermuteMaskMap(torch.autograd.Function):
         ctx.num_rows = num_rows
         ctx.probs_dtype = probs.dtype if probs is not None else None
         ctx.mark_non_differentiable(sorted_indices)
-        _remember_row_map(routing_map, num_rows, drop_and_pad, row_id_map)
+        _remember_row_map(routing_map, num_rows, drop_and_pad, row_id_map, sorted_flat, sorted_indices)
         return permuted, permuted_probs, sorted_indices
 
     @staticmethod
@@ -196,10 +219,25 @@ class MoeUnpermuteMaskMap(torch.autograd.Function):
         permuted_tokens = permuted_tokens.contiguous()
         num_experts = routing_map.size(1)
         num_rows, hidden = permuted_tokens.shape
-        row_id_map = _recall_row_map(routing_map, num_rows, drop_and_pad)
-        if row_id_map is None:
-            _, row_id_map, _, _ = routing_map_row_maps(routing_map, num_rows, drop_and_pad)
-            _remember_row_map(routing_map, num_rows, drop_and_pad, row_id_map)
+        kept = _recall_row_map(routing_map, num_rows, drop_and_pad)
+        own_indices = None
+        if kept is None:
+            _, row_id_map, sorted_flat, _ = routing_map_row_maps(routing_map, num_rows, drop_and_pad)
+            _remember_row_map(routing_map, num_rows, drop_and_pad, row_id_map, sorted_flat)
+        else:
+            row_id_map, sorted_flat, own_indices = kept
+        # The rows are gathered by the map that the mask gives.  ``sorted_indices`` must say the same: the torch path
+        # scatters row r to token sorted_indices[r] (unpermute_without_activation.py:54-62), so a re-ordered index
+        # would mean another result there.  The tensor that ``permute`` itself returned for this mask is known to
+        # agree; any other one is compared on the device (one read-back of a flag) unless
+        # MINDSPEED_AMD_CHECK_SORTED_INDICES=0.
+        if sorted_indices is not own_indices and _CHECK_SORTED_INDICES and not _tracing(sorted_indices):
+            expect = torch.div(sorted_flat.clamp(min=0), num_experts, rounding_mode="floor")
+            same = (sorted_indices.reshape(-1).to(expect.dtype) == expect) | (sorted_flat < 0)
+            if not bool(same.all()):
+                raise ValueError("sorted_indices is not the token order that routing_map gives (row r of permuted_tokens "
+                                 "belongs to the r-th set entry of routing_map in expert-major order): unpermute "
+                                 "recomputes the rows from routing_map and would silently ignore another order")
         if probs is not None:
             _lib.require_device(probs, "probs")
             if probs.shape != routing_map.shape:
@@ -208,21 +246,25 @@ class MoeUnpermuteMaskMap(torch.autograd.Function):
             _lib.dtype_code(probs.dtype, "probs")
             probs = probs.contiguous()          # used in their own dtype, e.g. fp32 beside bf16 tokens
         out = K.moe_token_unpermute(permuted_tokens, row_id_map, probs, num_tokens, num_experts)
-        ctx.save_for_backward(permuted_tokens if probs is not None else None, row_id_map, probs)
+        ctx.save_for_backward(permuted_tokens if probs is not None else None, row_id_map, probs, sorted_flat)
         ctx.num_tokens, ctx.num_experts, ctx.num_rows, ctx.hidden = num_tokens, num_experts, num_rows, hidden
+        ctx.all_rows_mapped = bool(drop_and_pad)      # every expert's capacity rows are filled (with padding entries)
         return out
 
     @staticmethod
     def backward(ctx, unpermuted_tokens_grad):
         if ctx.empty:   # permutation.py:104-105
             return unpermuted_tokens_grad, None, None, ctx.probs, None, None
-        permuted_tokens, row_id_map, probs = ctx.saved_tensors
+        permuted_tokens, row_id_map, probs, sorted_flat = ctx.saved_tensors
         grad_out = unpermuted_tokens_grad.contiguous()
-        # Every row has exactly one entry mapping to it.  Rows that nothing maps to exist only when the caller's
-        # row count exceeds the number of set mask entries; they belong to no expert and stay unwritten.
+        # Every mapped row has exactly one entry leading to it and is written by the gradient kernel.  Rows that
+        # nothing maps to exist only when the caller's row count exceeds the number of set mask entries; they are
+        # marked in sorted_flat and written as zeros (a launch whose workgroups all return at once when there are none).
         grad_permuted, grad_probs = K.moe_token_unpermute_grad(
             permuted_tokens if probs is not None else grad_out.new_empty(0), grad_out, row_id_map, probs,
             ctx.num_tokens, ctx.num_experts, ctx.num_rows)
+        if not ctx.all_rows_mapped:
+            K.zero_unmapped_rows(grad_permuted, sorted_flat)
         if probs is None or not ctx.needs_input_grad[3]:
             grad_probs = None
         return grad_permuted, None, None, grad_probs, None, None

@@ -16,7 +16,7 @@ over that average, next to the 8 TB/s HBM peak.  The ops:
     permute_grad    ms_moe_token_permute_grad     unweighted top-k gather
     unpermute_mask, unpermute_mask_grad, permute_mask_grad
                     the three gathers above driven by the routing-map form's row map (top-k = experts)
-    copy            ms_copy_bytes                 plain copy of the permuted rows, for orientation
+    copy            mb_copy_bytes (helper library) plain copy of the permuted rows, for orientation
 """
 from __future__ import annotations
 
@@ -25,7 +25,7 @@ import ctypes
 
 import torch
 
-from . import _lib, flop_counter
+from . import _lib, flop_counter, microbench_kernels
 
 HBM_PEAK_GBS = 8000.0
 
@@ -41,6 +41,7 @@ def measure(num_tokens=4096, hidden=4096, num_experts=8, topk=2, dtype=torch.bfl
         raise RuntimeError("permute_microbench needs a HIP device")
     dev = torch.device("cuda", 0) if device is None else device
     lib = _lib.load()
+    mb = microbench_kernels.load()
     T, H, E, K = num_tokens, hidden, num_experts, topk
     elem = torch.empty(0, dtype=dtype).element_size()
     code = _lib.dtype_code(dtype, "tokens")
@@ -107,7 +108,7 @@ def measure(num_tokens=4096, hidden=4096, num_experts=8, topk=2, dtype=torch.bfl
         "permute_mask_grad": (lambda b: lib.ms_moe_token_permute_grad(
             stream, P(b.perm), P(b.mask_map), T, E, H, code, rows, P(b.out)),
             flop_counter.permute_grad_bytes(T, K, H, elem) + T * (E - K) * 4),
-        "copy": (lambda b: lib.ms_copy_bytes(stream, P(b.perm), P(b.copy_dst), b.perm.numel() * elem),
+        "copy": (lambda b: mb.mb_copy_bytes(stream, P(b.perm), P(b.copy_dst), b.perm.numel() * elem),
                  2 * rows * H * elem),
     }
     result = {}

@@ -272,3 +272,75 @@ def test_row_map_is_remembered_on_the_mask(device):
     finally:
         M.routing_map_row_maps = real
     assert torch.equal(out1, out2) and torch.equal(out1, out3)
+
+
+@pytest.mark.parametrize("T,E,k,H,dtype", [(300, 8, 2, 256, torch.bfloat16), (300, 6, 2, 70, torch.float32),
+                                           (300, 900, 2, 32, torch.bfloat16)])
+def test_unpermute_gradient_has_no_unwritten_rows(T, E, k, H, dtype, device):
+    """A row count above the number of set entries: the rows of ``grad_permuted`` that nothing maps to are zeros, not
+    whatever the allocator handed out; the mapped rows are the oracle's."""
+    say("routing-map unpermute gradient, over-provisioned rows", T, E, k, H, dtype)
+    rmap, probs = make_map(T, E, k, seed=T + E + 1)
+    probs = probs.to(dtype)
+    gen = torch.Generator().manual_seed(3)
+    tokens = torch.randn(T, H, generator=gen).to(dtype)
+    gy = torch.randn(T, H, generator=gen).to(dtype)
+    nnz, extra = int(rmap.sum()), 53
+    rd, pd = rmap.to(device), probs.to(device)
+    perm, _, sidx = M.permute(tokens.to(device), rd, pd, num_out_tokens=nnz + extra, fused=True)
+    for with_probs in (True, False):
+        pin = perm.detach().clone().requires_grad_(True)
+        poison = torch.full((1 << 22,), float("nan"), device=device)
+        del poison
+        out = M.unpermute(pin, sidx, tokens.shape, probs=pd if with_probs else None, routing_map=rd, fused=True)
+        out.backward(gy.to(device))
+        torch.cuda.synchronize()
+        assert pin.grad.shape == (nnz + extra, H)
+        assert torch.count_nonzero(pin.grad[nnz:]) == 0 and not torch.isnan(pin.grad).any()
+        o_perm, _, o_sidx = O.permute_routing_map(tokens, rmap, probs)
+        o_in = o_perm.clone().requires_grad_(True)
+        O.unpermute_routing_map(o_in, o_sidx, tokens.shape, probs=probs if with_probs else None,
+                                routing_map=rmap).backward(gy)
+        assert rel_l2(pin.grad[:nnz], o_in.grad) <= TOL[dtype]
+
+
+def test_unpermute_checks_foreign_sorted_indices(device):
+    """``unpermute`` gathers by the map the mask gives.  The index tensor that ``permute`` returned for the mask is
+    trusted as it is; any other tensor is compared with that map on the device, and one that names another order
+    (which the torch path would follow, unpermute_without_activation.py:54-62) is refused instead of being ignored."""
+    T, E, k, H = 200, 8, 2, 64
+    rmap, probs = make_map(T, E, k, 321)
+    rd, pd = rmap.to(device), probs.to(device)
+    tokens = torch.randn(T, H, device=device).to(torch.bfloat16)
+    perm, _, sidx = M.permute(tokens, rd, pd, num_out_tokens=T * k, fused=True)
+    ref = M.unpermute(perm, sidx, tokens.shape, probs=pd, routing_map=rd, fused=True)
+    same = M.unpermute(perm, sidx.clone(), tokens.shape, probs=pd, routing_map=rd, fused=True)   # equal values: accepted
+    assert torch.equal(ref, same)
+    also = M.unpermute(perm, sidx.to(torch.int32), tokens.shape, probs=pd, routing_map=rd, fused=True)
+    assert torch.equal(ref, also)
+    swapped = sidx.clone()
+    swapped[[0, 1]] = swapped[[1, 0]] if swapped[0] != swapped[1] else swapped[[1, 0]] + 1
+    with pytest.raises(ValueError, match="token order"):
+        M.unpermute(perm, swapped, tokens.shape, probs=pd, routing_map=rd, fused=True)
+    with pytest.raises(ValueError, match="token order"):
+        M.unpermute(perm, torch.flip(sidx, [0]), tokens.shape, probs=pd, routing_map=rd.clone(), fused=True)
+
+
+def test_row_map_memory_follows_the_mask_storage(device):
+    """The remembered map is tied to the mask's version counter, storage address, shape and strides: a mask whose
+    storage was swapped under the same tensor object (``set_``), which leaves the version counter alone, is sorted
+    again."""
+    T, E, k, H = 128, 8, 2, 32
+    rmap, probs = make_map(T, E, k, 77)
+    other, _ = make_map(T, E, k, 78)
+    rd, pd = rmap.to(device), probs.to(device)
+    tokens = torch.randn(T, H, device=device).to(torch.bfloat16)
+    M.permute(tokens, rd, pd, num_out_tokens=T * k, fused=True)
+    assert M._recall_row_map(rd, T * k, False) is not None
+    version = rd._version
+    rd.set_(other.to(device))
+    assert rd._version == version or M._recall_row_map(rd, T * k, False) is None
+    assert M._recall_row_map(rd, T * k, False) is None
+    perm, _, sidx = M.permute(tokens, rd, None, num_out_tokens=T * k, fused=True)
+    o_perm, _, o_sidx = O.permute_routing_map(tokens.cpu(), other, None)
+    assert torch.equal(perm.cpu(), o_perm) and torch.equal(sidx.cpu(), o_sidx)

@@ -1,6 +1,7 @@
 """Host-side mirror of the reference interface: signatures, argument checks and
 error types, and the rule that nothing computes off the GPU.  No GPU needed."""
 import inspect
+import os
 
 import pytest
 import torch
@@ -264,11 +265,14 @@ def test_shapes_propagate_on_meta_tensors():
     assert xc.grad.shape == (T, H) and pc.grad.shape == (T,)
 
 
-def test_probe_sources_and_trace_build_are_wired():
-    """The hardware probes are listed by their runner, and the diagnostic (tile trace) build has its own output path."""
-    from mindspeed_amd import build
-    from mindspeed_amd.probes import __main__ as probes
+def test_trace_and_microbench_builds_are_wired():
+    """The diagnostic (tile trace) build and the measurement helpers have output paths of their own, and the plain copy
+    kernel is not part of the product's C ABI."""
+    from mindspeed_amd import _lib, build
 
-    assert probes.names() == ["issue_cost", "lds_rates", "mfma_power"]
     assert build.TRACE_LIB_PATH != build.LIB_PATH and build.TRACE_LIB_PATH.endswith("libmindspeed_amd_trace.so")
-    assert callable(build.build_trace)
+    assert build.MICROBENCH_LIB_PATH not in (build.LIB_PATH, build.TRACE_LIB_PATH)
+    assert callable(build.build_trace) and callable(build.build_microbench)
+    assert not any("copy" in name for name in _lib.EXPORTED_SYMBOLS)
+    header = open(os.path.join(os.path.dirname(build.HERE), "include", "mindspeed_amd.h")).read()
+    assert "ms_copy_bytes" not in header
