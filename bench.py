@@ -115,6 +115,25 @@ def cpu_baseline(cfg, budget_s=12.0):
         dtb = _cpu_layer_once(cfg, nb, torch.bfloat16)
         extra["bf16"] = {"value": round(nb / dtb, 2), "unit": "tokens/s", "cores": threads,
                          "sample": f"{nb} tokens, one forward+backward in bf16 ({dtb:.1f} s)"}
+    # the headline shape's forward pass whole, once: nothing extrapolated
+    if cfg["dtype"] == "bf16" and T * cfg["H"] * cfg["F"] <= 4096 * 4096 * 14336:
+        from oracle import moe_oracle as O
+        gen = torch.Generator().manual_seed(0)
+        H, E, F = cfg["H"], cfg["E"], cfg["F"]
+        xw = torch.randn(T, H, generator=gen)
+        # only the time is taken: the weights are a random block tiled to the full shape (drawing 1.4 G normal
+        # variates on one thread would take longer than the pass itself)
+        w1 = torch.randn(1, H, 2 * F // 8, generator=gen).mul_(0.02).repeat(E, 1, 8)
+        w2 = torch.randn(1, F // 8, H, generator=gen).mul_(0.02).repeat(E, 8, 1)
+        pw, idxw = make_routing(cfg, 0)
+        with torch.no_grad():
+            t0 = time.perf_counter()
+            O.moe_layer(xw, idxw, pw.float(), w1, w2)
+            dtw = time.perf_counter() - t0
+        del xw, w1, w2
+        extra["whole_forward"] = {"value": round(T / dtw, 1), "unit": "tokens/s", "cores": threads,
+                                  "sample": f"all {T} tokens of the workload, forward pass only (configs[1]), fp32, one "
+                                            f"run ({dtw:.1f} s): no extrapolation"}
     # configs[0], the reference's CPU-runnable case, whole (no extrapolation): median of five runs
     from mindspeed_amd.workloads import WORKLOADS
     small = WORKLOADS["plumbing"]

@@ -133,11 +133,42 @@ def require_device(t: torch.Tensor, what: str):
 
 
 def ptr(t):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    """Device address of a tensor as a plain int (ctypes converts it to the void* argument), None for no tensor."""
+    return None if t is None else t.data_ptr()
 
 
-def stream_ptr(device) -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+_raw_stream = torch._C._cuda_getCurrentRawStream
+
+
+def stream_ptr(device) -> int:
+    """The current stream of ``device`` as the integer handle the C ABI takes (a hipStream_t)."""
+    index = device.index
+    return _raw_stream(torch.cuda.current_device() if index is None else index)
+
+
+class _Guard:
+    """``with on(device):`` makes ``device`` current for the calls inside; free when it already is."""
+    __slots__ = ("index", "prev")
+
+    def __init__(self, device):
+        self.index = device.index
+
+    def __enter__(self):
+        self.prev = -1
+        if self.index is not None:
+            cur = torch.cuda.current_device()
+            if cur != self.index:
+                self.prev = cur
+                torch.cuda.set_device(self.index)
+        return self
+
+    def __exit__(self, *exc):
+        if self.prev >= 0:
+            torch.cuda.set_device(self.prev)
+        return False
+
+
+on = _Guard
 
 
 def workspace(nbytes: int, device) -> torch.Tensor:

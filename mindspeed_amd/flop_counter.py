@@ -86,20 +86,47 @@ def timing_active() -> bool:
     return _active is not None and _active.timing
 
 
-@contextlib.contextmanager
+class _NoOp:
+    __slots__ = ()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NOOP = _NoOp()
+
+
+class _Bracket:
+    __slots__ = ("rec", "name", "work", "unit", "device", "stream", "e0")
+
+    def __init__(self, rec, name, work, unit, device):
+        self.rec, self.name, self.work, self.unit, self.device = rec, name, work, unit, device
+
+    def __enter__(self):
+        self.e0 = None
+        if self.rec.timing:
+            self.stream = torch.cuda.current_stream(self.device)
+            self.e0 = torch.cuda.Event(enable_timing=True)
+            self.e0.record(self.stream)
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        e1 = None
+        if self.rec.timing:
+            e1 = torch.cuda.Event(enable_timing=True)
+            e1.record(self.stream)
+        if exc_type is None:
+            self.rec.calls.append((self.name, self.work() if callable(self.work) else self.work, self.unit, self.e0, e1))
+        return False
+
+
 def op(name, work, unit, device):
-    """Used by the ops around each C-ABI call; free when no Recorder is active."""
+    """Used by the ops around each C-ABI call: ``with op(...):``.  Free when no Recorder is active (``work`` may be a
+    callable, evaluated only when one is)."""
     rec = _active
     if rec is None:
-        yield
-        return
-    e0 = e1 = None
-    if rec.timing:
-        stream = torch.cuda.current_stream(device)
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-    yield
-    if rec.timing:
-        e1.record(stream)
-    rec.calls.append((name, work, unit, e0, e1))
+        return _NOOP
+    return _Bracket(rec, name, work, unit, device)

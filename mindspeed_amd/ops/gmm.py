@@ -17,7 +17,7 @@ import os
 import torch
 
 from .. import _lib, flop_counter
-from ._kernels import K
+from ._kernels import K, _plain
 from .npu_groupmatmul_add import npu_groupmatmul_add_fp32
 
 __all__ = ["npu_gmm", "npu_gmm_v2", "GMMFunction"]
@@ -419,14 +419,18 @@ def _npu_gmm_common(original_weight, x, weight, *, bias=None, group_list=None, g
         raise ValueError("group_list is required: the single-tensor (split_item=3) form needs group boundaries")
     if bias is not None and group_type != 0:
         raise ValueError("bias is supported with the split on rows (group_type 0) only")
+    # Plain device tensors in eager mode: the composite op's implementation directly (what the dispatcher would
+    # decompose to), without the boxing of a Python-registered op; anything that may want to see the call goes
+    # through the dispatcher.
+    direct = _plain((original_weight, x, weight, bias, group_list if isinstance(group_list, torch.Tensor) else None))
     if group_list_type == 0:
-        return torch.ops.mindspeed.npu_gmm(original_weight, x, weight, bias=bias, group_list=group_list,
-                                           group_type=group_type, gemm_fusion=gemm_fusion)
+        fn = _npu_gmm if direct else torch.ops.mindspeed.npu_gmm
     elif group_list_type == 1:
-        return torch.ops.mindspeed.npu_gmm_v2(original_weight, x, weight, bias=bias, group_list=group_list,
-                                              group_type=group_type, gemm_fusion=gemm_fusion)
+        fn = _npu_gmm_v2 if direct else torch.ops.mindspeed.npu_gmm_v2
     else:
         raise ValueError(f"group_list_type must be 0 or 1, but got {group_list_type}.")
+    return fn(original_weight, x, weight, bias=bias, group_list=group_list, group_type=group_type,
+              gemm_fusion=gemm_fusion)
 
 
 def npu_gmm(x, weight, *, bias=None, group_list=None, group_type=0, gemm_fusion=False, original_weight=None):
