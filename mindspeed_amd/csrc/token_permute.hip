@@ -286,23 +286,41 @@ __global__ __launch_bounds__(kSortBlockWaves * 64) void sort_small_kernel(
 }
 
 // ---- multi-block sort (large inputs): histogram, scan, scatter ----------------------
+// table[s][bin] = keys of `bin` in segment s.  One workgroup of 256 threads per segment: every thread requests all its
+// keys at once (unconditional loads from clamped positions) and counts them into the segment's LDS row with
+// fire-and-forget adds (a count does not depend on the order of its additions).  At 65536 positions in 64 segments
+// this takes a third of the time of one wavefront per segment matching its lanes' keys against each other, which left
+// the launch with 64 busy wavefronts on the whole chip.
+constexpr int kHistThreads = 256;
+constexpr int kHistKeysPerThread = 16;       // one pass over a segment of up to 4096 positions
 template <typename IdxT>
-__global__ __launch_bounds__(kHistWavesPerBlock * 64) void sort_hist_kernel(
+__global__ __launch_bounds__(kHistThreads) void sort_hist_kernel(
     const IdxT *__restrict__ idx, int n, int seg, int nseg, int nbins, int nbits, int *table) {
-    extern __shared__ int lds[];  // [kHistWavesPerBlock][nbins]
-    const int wave = threadIdx.x >> 6;
-    const int lane = threadIdx.x & 63;
-    const int s = blockIdx.x * kHistWavesPerBlock + wave;
-    int *row = lds + wave * nbins;
-    for (int e = lane; e < nbins; e += 64) row[e] = 0;
-    __builtin_amdgcn_wave_barrier();
-    if (s < nseg) {
-        const int begin = min(s * seg, n);
-        const int end = min(begin + seg, n);
-        wave_histogram(row, idx, begin, end, nbins, nbits);
-        __builtin_amdgcn_wave_barrier();
-        for (int e = lane; e < nbins; e += 64) table[static_cast<int64_t>(s) * nbins + e] = row[e];
+    extern __shared__ int lds[];  // [nbins]
+    (void)nbits;
+    const int s = blockIdx.x;
+    const int tid = threadIdx.x;
+    for (int e = tid; e < nbins; e += kHistThreads) lds[e] = 0;
+    const int begin = min(s * seg, n);
+    const int end = min(begin + seg, n);
+    __syncthreads();
+    // (one pass for segments of up to 4096 positions, which is all but inputs beyond 16 M positions)
+    for (int c = begin; c < end; c += kHistThreads * kHistKeysPerThread) {
+        IdxT raw[kHistKeysPerThread];
+#pragma unroll
+        for (int u = 0; u < kHistKeysPerThread; ++u) raw[u] = idx[min(c + u * kHistThreads + tid, end - 1)];
+#pragma unroll
+        for (int u = 0; u < kHistKeysPerThread; ++u) {
+            if (c + u * kHistThreads + tid < end) {
+                long long v = static_cast<long long>(raw[u]);
+                v = v < 0 ? 0 : v;
+                v = v >= nbins ? nbins - 1 : v;
+                __hip_atomic_fetch_add(&lds[static_cast<int>(v)], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
     }
+    __syncthreads();
+    for (int e = tid; e < nbins; e += kHistThreads) table[static_cast<int64_t>(s) * nbins + e] = lds[e];
 }
 
 __global__ __launch_bounds__(1024) void sort_scan_kernel(int *table, int nseg, int nbins,
@@ -1351,10 +1369,8 @@ inline SortPlan make_sort_plan(int64_t n, int64_t experts_hint) {
 template <typename IdxT>
 int launch_sort_offsets(hipStream_t stream, const SortPlan &p, const IdxT *idx, int64_t *tpe, int tpe_n, int *table,
                         bool scan = true) {
-    const int blocks = static_cast<int>(ceil_div(p.nseg, kHistWavesPerBlock));
-    const size_t lds = static_cast<size_t>(kHistWavesPerBlock) * p.nbins * sizeof(int);
-    hipLaunchKernelGGL(sort_hist_kernel<IdxT>, dim3(blocks), dim3(kHistWavesPerBlock * 64), lds, stream, idx, p.n,
-                       p.seg, p.nseg, p.nbins, p.nbits, table);
+    hipLaunchKernelGGL(sort_hist_kernel<IdxT>, dim3(p.nseg), dim3(kHistThreads), static_cast<size_t>(p.nbins) * sizeof(int),
+                       stream, idx, p.n, p.seg, p.nseg, p.nbins, p.nbits, table);
     MS_CHECK_LAUNCH("sort_hist_kernel");
     if (!scan) return MS_OK;
     hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(1024), 0, stream, table, p.nseg, p.nbins, tpe, tpe_n);
@@ -1512,13 +1528,21 @@ int launch_gather_combine(hipStream_t stream, const void *rows, const int32_t *m
 #define MS_GC_ARGS                                                                                                  \
     static_cast<const S *>(rows), map, static_cast<const PS *>(probs), static_cast<S *>(out), static_cast<int>(T),  \
         static_cast<int>(k), static_cast<int>(H), static_cast<int>(num_rows), rl.lanes
-    // many slots per token (the routing-map form has one per expert): list the valid ones first
-    const bool compact = k > 8 && rl.rows_per_block * k <= kCompactMaxLocal;
+    // many slots per token, or a map most of whose slots lead nowhere (the routing-map form has one slot per expert
+    // and only top-k of them set): list the valid ones first.  With at most two valid slots per token on average the
+    // listed rows are read like a top-2 map's, four vectors per slot in flight (measured on the 8-expert top-2 mask
+    // with buffers that do not fit the last-level cache: 26.0 -> 21 us; with all slots tested in place only the valid
+    // quarter of the eight-slot batch has loads in flight).
+    const bool sparse = k > 2 && 2 * num_rows <= T * k;
+    const bool compact = (k > 8 || sparse) && rl.rows_per_block * k <= kCompactMaxLocal;
+    const bool pairs = compact && num_rows <= 2 * T;
     const size_t lds = compact ? static_cast<size_t>(2) * rl.rows_per_block * k * sizeof(int) : 0;
     if (!vec_ok && compact) {
         hipLaunchKernelGGL((gather_combine_kernel<DT, PT, 1, 8, 2, true>), dim3(blocks), dim3(256), lds, stream, MS_GC_ARGS);
     } else if (!vec_ok) {
         hipLaunchKernelGGL((gather_combine_kernel<DT, PT, 1, 8, 2, false>), dim3(blocks), dim3(256), 0, stream, MS_GC_ARGS);
+    } else if (pairs) {
+        hipLaunchKernelGGL((gather_combine_kernel<DT, PT, VEC, 2, 4, true>), dim3(blocks), dim3(256), lds, stream, MS_GC_ARGS);
     } else if (compact) {
         hipLaunchKernelGGL((gather_combine_kernel<DT, PT, VEC, 8, 2, true>), dim3(blocks), dim3(256), lds, stream, MS_GC_ARGS);
     } else if (k <= 2) {
@@ -1546,12 +1570,17 @@ int launch_unpermute_grad(hipStream_t stream, const void *permuted, const void *
     static_cast<const S *>(permuted), static_cast<const S *>(gy), map, static_cast<const PS *>(probs),               \
         static_cast<S *>(gperm), static_cast<PS *>(gprobs), static_cast<int>(T), static_cast<int>(k),                \
         static_cast<int>(H), static_cast<int>(num_rows), rl.lanes
-    const bool compact = k > 8 && rl.rows_per_block * k <= kCompactMaxLocal;
+    // (the same choice as the gather's: list the valid slots of a many-slot or mostly empty map first)
+    const bool sparse = k > 2 && 2 * num_rows <= T * k;
+    const bool compact = (k > 8 || sparse) && rl.rows_per_block * k <= kCompactMaxLocal;
+    const bool pairs = compact && num_rows <= 2 * T;
     const size_t lds = compact ? static_cast<size_t>(3) * rl.rows_per_block * k * sizeof(int) : 0;
     if (!vec_ok && compact) {
         hipLaunchKernelGGL((unpermute_grad_kernel<DT, PT, 1, 4, 4, true>), grid, dim3(256), lds, stream, MS_UG_ARGS);
     } else if (!vec_ok) {
         hipLaunchKernelGGL((unpermute_grad_kernel<DT, PT, 1, 4, 4, false>), grid, dim3(256), 0, stream, MS_UG_ARGS);
+    } else if (pairs) {
+        hipLaunchKernelGGL((unpermute_grad_kernel<DT, PT, VEC, 2, 4, true>), grid, dim3(256), lds, stream, MS_UG_ARGS);
     } else if (compact) {
         hipLaunchKernelGGL((unpermute_grad_kernel<DT, PT, VEC, 4, 2, true>), grid, dim3(256), lds, stream, MS_UG_ARGS);
     } else if (k <= 2) {
