@@ -63,6 +63,25 @@ def measured_traffic(workload, kernel):
     return data.get("bytes_per_launch", {}).get(workload, {}).get(kernel)
 
 
+IN_LAYER_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "permute_family_in_layer.json")
+
+
+def measured_in_layer_durations(workload):
+    """Kernel durations of the HBM-bound ops inside the layer step as rocprofv3 --kernel-trace read them (the event
+    brackets under `kernels` include a few microseconds that are not the kernel), from the tracked summary that
+    `python -m mindspeed_amd.profile_tools in-layer` wrote: only if it was measured on the kernel sources as they are
+    now, else None."""
+    from mindspeed_amd.build import source_hash
+    try:
+        with open(IN_LAYER_FILE) as fh:
+            data = json.load(fh)
+    except (OSError, ValueError):
+        return None
+    if data.get("build") != source_hash():
+        return None
+    return data.get("kernels", {}).get(workload)
+
+
 def _cpu_layer_once(cfg, sample, dtype=torch.float32):
     from oracle import moe_oracle as O
 
@@ -434,6 +453,26 @@ def main():
             "note": "back-to-back launches through the C ABI, event-timed over 200 launches per op; algorithmic bytes "
                     "over the average, against the 8 TB/s HBM peak and against the plain copy kernel in the same mode",
             "cold_buffer_sets": cold_sets, "warm": warm, "cold": cold}
+        if args.workload == "mixtral":
+            # the same at the shapes of the other two BASELINE configurations (index form and routing-map form of the
+            # four ops, and the copy), fraction of the 8 TB/s peak and of the copy: their buffers exceed the
+            # last-level cache already with one set, the rotation ("cold") adds a second or third
+            brief = ("permute", "permute_mask", "unpermute", "unpermute_mask", "unpermute_grad", "permute_grad", "copy")
+            for name in ("deepseek", "qwen"):
+                o = WORKLOADS[name]
+                oshape = (o["T"], o["H"], o["E"], o["K"], torch.bfloat16)
+                tables = {"one_buffer_set": measure_permute_family(*oshape, device=device, iters=100),
+                          "cold": measure_permute_family(*oshape, device=device, iters=100,
+                                                         sets=sets_for_cold(o["T"], o["H"], o["K"]))}
+                result["permute_family"][name] = {
+                    "shape": f"{o['T']} tokens x hidden {o['H']}, {o['E']} experts, top-{o['K']}",
+                    **{mode: {k: {"avg_us": t[k]["avg_us"], "frac_of_hbm_peak": t[k]["frac_of_hbm_peak"],
+                                  "frac_of_copy": round(t[k]["gbs"] / t["copy"]["gbs"], 3)} for k in brief}
+                       for mode, t in tables.items()}}
+                torch.cuda.empty_cache()
+        in_layer = measured_in_layer_durations(args.workload)
+        if in_layer is not None:
+            result["permute_family"]["in_layer_rocprofv3"] = in_layer
 
     others = {}
 

@@ -1,12 +1,17 @@
 """Grouped-matmul launches of the Mixtral-shape expert MLP in isolation.
 
-    python -m mindspeed_amd.gmm_microbench [--mode fwd1|fwd2|dx1|dx2|dw1|dw2|dw1acc|dw2acc|library] [--data randn|small|ones|zeros]
+    python -m mindspeed_amd.gmm_microbench [--mode fwd1|fwd2|dx1|dx2|dw1|dw2|dw1acc|dw2acc|library|library_nt|library_tn|all]
+                                           [--data randn|small|ones|zeros]
                                            [--dtype bf16|fp16|fp32] [--counts 988,1074,...] [--iters 20] [--warmup 20]
 
 ``fwd1`` / ``dx1`` / ``dw1`` are the forward, dX and dW products of the first matmul
 (``[T, H] x [E, H, 2F]``), ``fwd2`` / ``dx2`` / ``dw2`` those of the second (``[T, F] x [E, F, H]``);
 ``dw1acc`` / ``dw2acc`` are the weight gradients added in place to an fp32 buffer;
-``library`` runs ``torch.bmm`` on the fc1-forward shape as E dense products, for orientation.
+``library`` runs ``torch.bmm`` on the fc1-forward shape as E dense products, for orientation, ``library_nt`` /
+``library_tn`` the same library on the operand layouts of the dX (weight read transposed) and dW (activations read
+transposed) products of that matmul (equal groups only).  ``all`` launches the six products one after the other,
+``--iters`` launches each and no warm-up, in the fixed order fwd1 fwd2 dx1 dx2 dw1 dw2: the form to put under
+``rocprofv3 --pmc`` (``python -m mindspeed_amd.profile_tools products`` reads the counters back per product).
 ``--data`` sets the operand values only (the rate of the matrix cores on this board depends on them);
 ``--counts`` gives the rows per expert (default: equal shares).  Prints milliseconds per launch and TFLOP/s.
 """
@@ -21,7 +26,7 @@ from .ops.gmm import gmm_raw
 
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--mode", default="fwd1", choices=["fwd1", "fwd2", "dx1", "dx2", "dw1", "dw2", "dw1acc", "dw2acc", "library"])
+    ap.add_argument("--mode", default="fwd1", choices=["fwd1", "fwd2", "dx1", "dx2", "dw1", "dw2", "dw1acc", "dw2acc", "library", "library_nt", "library_tn", "all"])
     ap.add_argument("--data", default="randn", choices=["randn", "small", "ones", "zeros"])
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32"], help="operand dtype")
     ap.add_argument("--iters", type=int, default=20)
@@ -54,6 +59,23 @@ def main():
             return torch.randint(-2, 3, shape, generator=gen, device=dev).to(bf)
         return torch.randn(*shape, generator=gen, device=dev).to(bf)
 
+    if a.mode == "all":
+        x1, w1, dy1 = operand(T, H), operand(E, H, 2 * F), operand(T, 2 * F)
+        x2, w2, dy2 = operand(T, F), operand(E, F, H), operand(T, H)
+        products = [("fwd1", lambda: gmm_raw(x1, w1, counts, 0, 1)), ("fwd2", lambda: gmm_raw(x2, w2, counts, 0, 1)),
+                    ("dx1", lambda: gmm_raw(dy1, w1.transpose(1, 2), counts, 0, 1)),
+                    ("dx2", lambda: gmm_raw(dy2, w2.transpose(1, 2), counts, 0, 1)),
+                    ("dw1", lambda: gmm_raw(x1.t(), dy1, counts, 2, 1)), ("dw2", lambda: gmm_raw(x2.t(), dy2, counts, 2, 1))]
+        torch.cuda.synchronize()
+        for name, fn in products:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(a.iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            print(f"{name} ({a.data}): {e0.elapsed_time(e1) / a.iters:.4f} ms per launch over {a.iters} launches", flush=True)
+        return
     if a.mode == "fwd1":
         x, w = operand(T, H), operand(E, H, 2 * F)
         fn, flops = (lambda: gmm_raw(x, w, counts, 0, 1)), 2 * T * H * 2 * F
@@ -78,6 +100,12 @@ def main():
         x, dy = (operand(T, H), operand(T, 2 * F)) if a.mode == "dw1acc" else (operand(T, F), operand(T, H))
         grad = torch.zeros(E, x.size(1), dy.size(1), device=dev, dtype=torch.float32)
         fn, flops = (lambda: gmm_raw(x.t(), dy, counts, 2, 1, out=grad, accumulate=True)), 2 * T * x.size(1) * dy.size(1)
+    elif a.mode == "library_nt":        # dX of fc1: dy [E, M, 2F] x (w [E, H, 2F])^T
+        dy, w = operand(E, T // E, 2 * F), operand(E, H, 2 * F)
+        fn, flops = (lambda: torch.bmm(dy, w.transpose(1, 2))), 2 * T * H * 2 * F
+    elif a.mode == "library_tn":        # dW of fc1: (x [E, M, H])^T x dy [E, M, 2F]
+        x, dy = operand(E, T // E, H), operand(E, T // E, 2 * F)
+        fn, flops = (lambda: torch.bmm(x.transpose(1, 2), dy)), 2 * T * H * 2 * F
     else:
         x, w = operand(E, T // E, H), operand(E, H, 2 * F)
         fn, flops = (lambda: torch.bmm(x, w)), 2 * T * H * 2 * F

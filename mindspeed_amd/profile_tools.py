@@ -1,7 +1,9 @@
 """Measurement helpers behind the figures under ``profiles/``.
 
     python -m mindspeed_amd.profile_tools traffic --fetch F.csv --write W.csv [--workload mixtral] [--out FILE.json]
-    python -m mindspeed_amd.profile_tools counters CSV [CSV ...]
+    python -m mindspeed_amd.profile_tools counters [--all] CSV [CSV ...]
+    python -m mindspeed_amd.profile_tools in-layer --stats KERNEL_STATS.csv [--workload mixtral] [--out FILE.json]
+    python -m mindspeed_amd.profile_tools products --csv COUNTERS.csv [--iters 3]
     python -m mindspeed_amd.profile_tools power [--seconds 4] [--modes fwd1,dx1,dw1,library] [--data randn,zeros]
     MINDSPEED_AMD_LIB=mindspeed_amd/libmindspeed_amd_trace.so python -m mindspeed_amd.profile_tools timeline [--modes ...] [--data ...]
 
@@ -11,7 +13,12 @@ among the dispatches), scales the counters by what they read for that copy, prin
 kernel of the library and, with ``--out``, records the grouped-matmul figures together with the hash of the kernel
 sources they belong to (``bench.py`` reports them as ``roofline.traffic`` as long as that hash is unchanged).
 
-``counters`` prints per-kernel averages of whatever counters the given files hold.
+``counters`` prints per-kernel averages of whatever counters the given files hold (this library's kernels only) and
+the ratios derived from them: MFMA busy share, LDS-wait and any-wait share of the wavefront cycles, LDS bank conflicts
+per LDS instruction cycle, L2 hit rate.
+
+``in-layer`` turns the kernel statistics of a ``rocprofv3 --kernel-trace --stats`` run of ``bench.py`` into the
+durations and HBM-roofline fractions of the permute / unpermute / SwiGLU kernels inside the layer step.
 
 ``power`` runs one grouped-matmul launch of the Mixtral-shape expert MLP back to back for a few seconds per
 (product, operand values) pair while a thread samples the board's power draw and shader clock from the amdgpu
@@ -111,7 +118,15 @@ def cmd_traffic(args):
         print(f"\nrecorded {record} for build {build} in {args.out}")
 
 
+def _own_kernel(name: str) -> bool:
+    """Kernels of this library (everything else in a trace is torch's own: fills, copies, random numbers)."""
+    return not name.startswith(("at::", "__amd", "rocclr")) and "at::native" not in name
+
+
 def cmd_counters(args):
+    """Per-kernel averages of the counters in the given files, this library's kernels only, and below them the ratios
+    they are collected for."""
+    merged = collections.defaultdict(dict)
     for path in args.files:
         agg = collections.defaultdict(lambda: collections.defaultdict(list))
         with open(path, newline="") as fh:
@@ -119,8 +134,101 @@ def cmd_counters(args):
                 agg[short_name(row["Kernel_Name"])][row["Counter_Name"]].append(float(row["Counter_Value"]))
         print(f"# {os.path.basename(path)}")
         for kernel, counters in agg.items():
+            if not _own_kernel(kernel) or (not args.all and "gmm16" not in kernel):
+                continue
             for counter, vals in counters.items():
-                print(f"{kernel[:90]:90s} {counter:28s} dispatches {len(vals):5d}  avg {sum(vals) / len(vals):16.1f}")
+                avg = sum(vals) / len(vals)
+                merged[kernel][counter] = avg
+                print(f"{kernel[:70]:70s} {counter:28s} dispatches {len(vals):5d}  avg {avg:16.1f}")
+    print("\n# derived (averages per dispatch)")
+    print(f"{'kernel':70s} {'MFMA busy':>10s} {'LDS wait':>10s} {'any wait':>10s} {'LDS bank confl.':>16s} {'L2 hit rate':>12s}")
+    for kernel, c in merged.items():
+        def ratio(num, den, scale=1.0):
+            return f"{c[num] / (scale * c[den]):.3f}" if num in c and den in c and c[den] else "-"
+        hit = f"{c['TCC_HIT_sum'] / (c['TCC_HIT_sum'] + c['TCC_MISS_sum']):.3f}" if "TCC_HIT_sum" in c and "TCC_MISS_sum" in c else "-"
+        # SQ_WAVE_CYCLES counts in units of 4 clocks per wavefront, the busy / wait counters in clocks
+        print(f"{kernel[:70]:70s} {ratio('SQ_VALU_MFMA_BUSY_CYCLES', 'SQ_WAVE_CYCLES', 4.0):>10s} "
+              f"{ratio('SQ_WAIT_INST_LDS', 'SQ_WAVE_CYCLES', 4.0):>10s} {ratio('SQ_WAIT_INST_ANY', 'SQ_WAVE_CYCLES', 4.0):>10s} "
+              f"{ratio('SQ_LDS_BANK_CONFLICT', 'SQ_ACTIVE_INST_LDS'):>16s} {hit:>12s}")
+
+
+def cmd_products(args):
+    """Per-product L2 counters of `python -m mindspeed_amd.gmm_microbench --mode all --iters N` run under
+    `rocprofv3 --pmc TCC_HIT_sum TCC_MISS_sum TCC_EA0_RDREQ_sum TCC_EA0_WRREQ_sum`: the grouped-matmul dispatches come in
+    the order fwd1 fwd2 dx1 dx2 dw1 dw2, N of each; the first of each product is left out of the average.  Reads from
+    the fabric are 128-byte requests (one L2 line), writes 64-byte ones (checked on kernels of known traffic)."""
+    rows = collections.OrderedDict()
+    with open(args.csv, newline="") as fh:
+        for row in csv.DictReader(fh):
+            if "gmm16_fast_kernel" in row["Kernel_Name"]:
+                rows.setdefault(int(row["Dispatch_Id"]), {})[row["Counter_Name"]] = float(row["Counter_Value"])
+    ids = sorted(rows)
+    names = ("fwd1", "fwd2", "dx1", "dx2", "dw1", "dw2")
+    if len(ids) != len(names) * args.iters:
+        raise SystemExit(f"expected {len(names) * args.iters} grouped-matmul dispatches, found {len(ids)}")
+    print(f"{'product':8s} {'fabric reads GB':>16s} {'fabric writes GB':>17s} {'L2 hit rate':>12s}")
+    for i, name in enumerate(names):
+        grp = [rows[j] for j in ids[i * args.iters:(i + 1) * args.iters]][1 if args.iters > 1 else 0:]
+        avg = {k: sum(g[k] for g in grp) / len(grp) for k in grp[0]}
+        hit = avg["TCC_HIT_sum"] / (avg["TCC_HIT_sum"] + avg["TCC_MISS_sum"])
+        print(f"{name:8s} {avg['TCC_EA0_RDREQ_sum'] * 128 / 1e9:16.2f} {avg['TCC_EA0_WRREQ_sum'] * 64 / 1e9:17.2f} {hit:12.3f}")
+
+
+# kernels of the HBM-bound ops inside the layer step: name fragment -> (label, algorithmic bytes of one launch)
+def _in_layer_ops(cfg):
+    from . import flop_counter
+    T, K, H, F = cfg["T"], cfg["K"], cfg["H"], cfg["F"]
+    elem = 2 if cfg["dtype"] == "bf16" else 4
+    rows = T * K
+    return {
+        "permute_fused_kernel": ("permute", flop_counter.permute_bytes(T, K, H, elem, 8)),
+        "permute_fused_bins_kernel": ("permute", flop_counter.permute_bytes(T, K, H, elem, 8)),
+        "permute_scatter_rows_kernel": ("permute (rows launch; the histogram launch is listed by itself)",
+                                        flop_counter.permute_bytes(T, K, H, elem, 8)),
+        "sort_hist_kernel": ("permute (histogram launch)", rows * 8),
+        "gather_combine_kernel": ("unpermute forward and permute backward (one kernel, averaged)",
+                                  flop_counter.unpermute_bytes(T, K, H, elem)),
+        "unpermute_grad_kernel": ("unpermute backward", flop_counter.unpermute_grad_bytes(T, K, H, elem)),
+        "swiglu_kernel": ("SwiGLU", flop_counter.swiglu_bytes(rows, F, elem)),
+        "swiglu_grad_kernel": ("SwiGLU backward", flop_counter.swiglu_bytes(rows, F, elem, True)),
+    }
+
+
+def cmd_in_layer(args):
+    """Durations of the HBM-bound kernels inside the layer step from a rocprofv3 --kernel-trace --stats run of bench.py
+    (the `*_kernel_stats.csv`), as fractions of the 8 TB/s peak of their algorithmic bytes."""
+    from .build import source_hash
+    from .workloads import WORKLOADS
+
+    ops = _in_layer_ops(WORKLOADS[args.workload])
+    found = {}
+    with open(args.stats, newline="") as fh:
+        for row in csv.DictReader(fh):
+            name = short_name(row["Name"])
+            for frag, (label, nbytes) in ops.items():
+                if name.startswith(frag + "<") or name == frag:
+                    us = float(row["AverageNs"]) / 1e3
+                    found[frag] = {"op": label, "calls": int(row["Calls"]), "avg_us": round(us, 2),
+                                   "bytes_per_launch": int(nbytes), "gbs": round(nbytes / us / 1e3, 1),
+                                   "frac_of_hbm_peak": round(nbytes / us / 1e3 / 8000.0, 4)}
+    print(f"{'kernel':30s} {'calls':>6s} {'avg_us':>9s} {'MB':>8s} {'GB/s':>8s} {'of 8 TB/s':>10s}  op")
+    for frag, r in found.items():
+        print(f"{frag:30s} {r['calls']:6d} {r['avg_us']:9.2f} {r['bytes_per_launch'] / 1e6:8.1f} {r['gbs']:8.1f} "
+              f"{r['frac_of_hbm_peak']:10.3f}  {r['op']}")
+    if args.out:
+        data = {}
+        if os.path.exists(args.out):
+            with open(args.out) as fh:
+                data = json.load(fh)
+        build = source_hash()
+        if data.get("build") != build:
+            data = {"build": build, "what": "rocprofv3 --kernel-trace --stats durations of the HBM-bound kernels inside "
+                                            "the layer step (bench.py), algorithmic bytes over the average", "kernels": {}}
+        data["kernels"][args.workload] = found
+        with open(args.out, "w") as fh:
+            json.dump(data, fh, indent=1, sort_keys=True)
+            fh.write("\n")
+        print(f"\nrecorded for build {build} in {args.out}")
 
 
 # ---- power / clock ---------------------------------------------------------------------------------------------
@@ -359,6 +467,14 @@ def main():
     t.add_argument("--out", default="")
     c = sub.add_parser("counters")
     c.add_argument("files", nargs="+")
+    c.add_argument("--all", action="store_true", help="every kernel of the library, not only the grouped matmuls")
+    pr = sub.add_parser("products")
+    pr.add_argument("--csv", required=True, help="the *_counter_collection.csv of the rocprofv3 --pmc run")
+    pr.add_argument("--iters", type=int, default=3)
+    il = sub.add_parser("in-layer")
+    il.add_argument("--stats", required=True, help="the *_kernel_stats.csv of a rocprofv3 --kernel-trace --stats run")
+    il.add_argument("--workload", default="mixtral")
+    il.add_argument("--out", default="")
     w = sub.add_parser("power")
     w.add_argument("--seconds", type=float, default=4.0)
     w.add_argument("--modes", default="fwd1,dx1,dw1,library")
@@ -368,7 +484,8 @@ def main():
     tl.add_argument("--data", default="randn,zeros")
     tl.add_argument("--counts", default="", help="comma-separated rows per expert instead of eight equal groups")
     args = ap.parse_args()
-    {"traffic": cmd_traffic, "counters": cmd_counters, "power": cmd_power, "timeline": cmd_timeline}[args.cmd](args)
+    {"traffic": cmd_traffic, "counters": cmd_counters, "power": cmd_power, "timeline": cmd_timeline,
+     "in-layer": cmd_in_layer, "products": cmd_products}[args.cmd](args)
 
 
 if __name__ == "__main__":
