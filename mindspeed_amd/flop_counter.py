@@ -47,7 +47,9 @@ def permute_grad_bytes(num_tokens, topk, hidden, elem, rows=None):
 
 
 def swiglu_bytes(rows, ffn, elem, backward=False):
-    return rows * ffn * elem * (6 if backward else 3)
+    """Forward: read gate and up, write the product (3 arrays of rows x ffn).  Backward: read gate, up and the
+    incoming gradient, write both halves of the input gradient (5)."""
+    return rows * ffn * elem * (5 if backward else 3)
 
 
 class Recorder:

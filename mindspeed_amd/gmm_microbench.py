@@ -1,15 +1,15 @@
 """Grouped-matmul launches of the Mixtral-shape expert MLP in isolation.
 
-    python -m mindspeed_amd.gmm_microbench [--mode fwd1|fwd2|dx1|dx2|dw1|dw2|dw1acc|dw2acc|library|library_nt|library_tn|all]
+    python -m mindspeed_amd.gmm_microbench [--mode fwd1|fwd2|dx1|dx2|dw1|dw2|dw1acc|dw2acc|library|all]
                                            [--data randn|small|ones|zeros]
                                            [--dtype bf16|fp16|fp32] [--counts 988,1074,...] [--iters 20] [--warmup 20]
 
 ``fwd1`` / ``dx1`` / ``dw1`` are the forward, dX and dW products of the first matmul
 (``[T, H] x [E, H, 2F]``), ``fwd2`` / ``dx2`` / ``dw2`` those of the second (``[T, F] x [E, F, H]``);
 ``dw1acc`` / ``dw2acc`` are the weight gradients added in place to an fp32 buffer;
-``library`` runs ``torch.bmm`` on the fc1-forward shape as E dense products, for orientation, ``library_nt`` /
-``library_tn`` the same library on the operand layouts of the dX (weight read transposed) and dW (activations read
-transposed) products of that matmul (equal groups only).  ``all`` launches the six products one after the other,
+``library`` runs ``torch.bmm`` on the fc1-forward shape as E dense products, for orientation (contiguous operands
+only: a run of this program's loop with ``torch.bmm`` on transposed views of these shapes ended in a GPU memory fault
+inside the vendor library's launches, so those layouts are not offered).  ``all`` launches the six products one after the other,
 ``--iters`` launches each and no warm-up, in the fixed order fwd1 fwd2 dx1 dx2 dw1 dw2: the form to put under
 ``rocprofv3 --pmc`` (``python -m mindspeed_amd.profile_tools products`` reads the counters back per product).
 ``--data`` sets the operand values only (the rate of the matrix cores on this board depends on them);
@@ -26,7 +26,7 @@ from .ops.gmm import gmm_raw
 
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--mode", default="fwd1", choices=["fwd1", "fwd2", "dx1", "dx2", "dw1", "dw2", "dw1acc", "dw2acc", "library", "library_nt", "library_tn", "all"])
+    ap.add_argument("--mode", default="fwd1", choices=["fwd1", "fwd2", "dx1", "dx2", "dw1", "dw2", "dw1acc", "dw2acc", "library", "all"])
     ap.add_argument("--data", default="randn", choices=["randn", "small", "ones", "zeros"])
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32"], help="operand dtype")
     ap.add_argument("--iters", type=int, default=20)
@@ -100,12 +100,6 @@ def main():
         x, dy = (operand(T, H), operand(T, 2 * F)) if a.mode == "dw1acc" else (operand(T, F), operand(T, H))
         grad = torch.zeros(E, x.size(1), dy.size(1), device=dev, dtype=torch.float32)
         fn, flops = (lambda: gmm_raw(x.t(), dy, counts, 2, 1, out=grad, accumulate=True)), 2 * T * x.size(1) * dy.size(1)
-    elif a.mode == "library_nt":        # dX of fc1: dy [E, M, 2F] x (w [E, H, 2F])^T
-        dy, w = operand(E, T // E, 2 * F), operand(E, H, 2 * F)
-        fn, flops = (lambda: torch.bmm(dy, w.transpose(1, 2))), 2 * T * H * 2 * F
-    elif a.mode == "library_tn":        # dW of fc1: (x [E, M, H])^T x dy [E, M, 2F]
-        x, dy = operand(E, T // E, H), operand(E, T // E, 2 * F)
-        fn, flops = (lambda: torch.bmm(x.transpose(1, 2), dy)), 2 * T * H * 2 * F
     else:
         x, w = operand(E, T // E, H), operand(E, H, 2 * F)
         fn, flops = (lambda: torch.bmm(x, w)), 2 * T * H * 2 * F

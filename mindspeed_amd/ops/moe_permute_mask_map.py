@@ -106,25 +106,34 @@ def _remember_row_map(routing_map, num_rows, drop_and_pad, row_id_map, sorted_fl
         kept = (state, {})
         routing_map._ms_row_maps = kept
     maps = kept[1]
+    # (the last element: index tensors known to agree with the map, as weak references with their version counters)
+    known = [] if sorted_indices is None else [(weakref.ref(sorted_indices), sorted_indices._version)]
     maps[(int(num_rows), bool(drop_and_pad))] = (row_id_map, sorted_flat, torch.cuda.current_stream(routing_map.device),
-                                                 None if sorted_indices is None else weakref.ref(sorted_indices))
+                                                 known)
     while len(maps) > _ROW_MAPS_KEPT:
         maps.pop(next(iter(maps)))
 
 
 def _recall_row_map(routing_map, num_rows, drop_and_pad):
-    """``(row_id_map, sorted_flat, sorted_indices or None)`` of an earlier ``permute`` of this very mask, or None."""
+    """``(row_id_map, sorted_flat, known index tensors)`` of an earlier ``permute`` of this very mask, or None."""
     kept = getattr(routing_map, "_ms_row_maps", None)
     if not _ROW_MAP_CACHE or kept is None or kept[0] != _mask_state(routing_map):
         return None
     hit = kept[1].get((int(num_rows), bool(drop_and_pad)))
     if hit is None:
         return None
-    row_id_map, sorted_flat, stream, own = hit
+    row_id_map, sorted_flat, stream, known = hit
     now = torch.cuda.current_stream(routing_map.device)
     if now != stream:
         now.wait_stream(stream)          # everything queued on the producing stream so far, the map's kernel included
-    return row_id_map, sorted_flat, (own() if own is not None else None)
+    return row_id_map, sorted_flat, known
+
+
+def _is_known(known, sorted_indices) -> bool:
+    for ref, version in known:
+        if ref() is sorted_indices and version == sorted_indices._version:
+            return True
+    return False
 
 
 def _tracing(t):
@@ -220,24 +229,27 @@ class MoeUnpermuteMaskMap(torch.autograd.Function):
         num_experts = routing_map.size(1)
         num_rows, hidden = permuted_tokens.shape
         kept = _recall_row_map(routing_map, num_rows, drop_and_pad)
-        own_indices = None
         if kept is None:
             _, row_id_map, sorted_flat, _ = routing_map_row_maps(routing_map, num_rows, drop_and_pad)
             _remember_row_map(routing_map, num_rows, drop_and_pad, row_id_map, sorted_flat)
-        else:
-            row_id_map, sorted_flat, own_indices = kept
+            kept = _recall_row_map(routing_map, num_rows, drop_and_pad)
+        known = kept[2] if kept is not None else []
+        if kept is not None:
+            row_id_map, sorted_flat = kept[0], kept[1]
         # The rows are gathered by the map that the mask gives.  ``sorted_indices`` must say the same: the torch path
         # scatters row r to token sorted_indices[r] (unpermute_without_activation.py:54-62), so a re-ordered index
         # would mean another result there.  The tensor that ``permute`` itself returned for this mask is known to
-        # agree; any other one is compared on the device (one read-back of a flag) unless
-        # MINDSPEED_AMD_CHECK_SORTED_INDICES=0.
-        if sorted_indices is not own_indices and _CHECK_SORTED_INDICES and not _tracing(sorted_indices):
+        # agree; any other one is compared on the device once (one read-back of a flag; a tensor that passed is
+        # remembered beside the map) unless MINDSPEED_AMD_CHECK_SORTED_INDICES=0.
+        if _CHECK_SORTED_INDICES and not _tracing(sorted_indices) and not _is_known(known, sorted_indices):
             expect = torch.div(sorted_flat.clamp(min=0), num_experts, rounding_mode="floor")
             same = (sorted_indices.reshape(-1).to(expect.dtype) == expect) | (sorted_flat < 0)
             if not bool(same.all()):
                 raise ValueError("sorted_indices is not the token order that routing_map gives (row r of permuted_tokens "
                                  "belongs to the r-th set entry of routing_map in expert-major order): unpermute "
                                  "recomputes the rows from routing_map and would silently ignore another order")
+            known.append((weakref.ref(sorted_indices), sorted_indices._version))
+            del known[:-4]
         if probs is not None:
             _lib.require_device(probs, "probs")
             if probs.shape != routing_map.shape:

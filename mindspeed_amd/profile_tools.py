@@ -4,7 +4,7 @@
     python -m mindspeed_amd.profile_tools counters [--all] CSV [CSV ...]
     python -m mindspeed_amd.profile_tools in-layer --stats KERNEL_STATS.csv [--workload mixtral] [--out FILE.json]
     python -m mindspeed_amd.profile_tools products --csv COUNTERS.csv [--iters 3]
-    python -m mindspeed_amd.profile_tools power [--seconds 4] [--modes fwd1,dx1,dw1,library] [--data randn,zeros]
+    python -m mindspeed_amd.profile_tools power [--seconds 4] [--modes fwd1,dx1,dw1] [--data randn,zeros]
     MINDSPEED_AMD_LIB=mindspeed_amd/libmindspeed_amd_trace.so python -m mindspeed_amd.profile_tools timeline [--modes ...] [--data ...]
 
 ``traffic`` reads the ``*_counter_collection.csv`` files of two ``rocprofv3 --pmc`` runs of ``bench.py`` (one with
@@ -52,7 +52,7 @@ GEMM_KEYS = {  # first template arguments <dtype, A reduction-contiguous, B redu
 
 
 def short_name(name: str) -> str:
-    name = name.replace("void ", "").replace("ms::(anonymous namespace)::", "")
+    name = name.replace("void ", "").replace("ms::(anonymous namespace)::", "").replace("(anonymous namespace)::", "")
     name = re.sub(r"\(.*$", "", name)
     return name.replace("(ms::OutMode)", "").replace("(int)", "")
 
@@ -477,7 +477,7 @@ def main():
     il.add_argument("--out", default="")
     w = sub.add_parser("power")
     w.add_argument("--seconds", type=float, default=4.0)
-    w.add_argument("--modes", default="fwd1,dx1,dw1,library")
+    w.add_argument("--modes", default="fwd1,dx1,dw1")
     w.add_argument("--data", default="randn,small,zeros")
     tl = sub.add_parser("timeline")
     tl.add_argument("--modes", default="fwd1,dx1,dw1")

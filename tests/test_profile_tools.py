@@ -97,3 +97,77 @@ def test_tracked_traffic_profile_belongs_to_these_sources():
     import bench
     for kernel in ("gmm_fwd", "gmm_dx", "gmm_dw"):
         assert bench.measured_traffic("mixtral", kernel) == data["bytes_per_launch"]["mixtral"][kernel] > 1e9
+
+
+DW = "void ms::(anonymous namespace)::gmm16_fast_kernel<0, false, false, 0, false>(ms::GmmArgs)"
+
+
+def test_counters_prints_the_derived_ratios(tmp_path):
+    """MFMA busy = busy clocks / (4 x wave cycles), L2 hit rate = hits / (hits + misses); torch's own kernels are left out."""
+    sq, tcc = tmp_path / "q.csv", tmp_path / "t.csv"
+    with open(sq, "w") as fh:
+        fh.write(HEADER)
+        for i, (k, c, v) in enumerate([(FWD, "SQ_WAVE_CYCLES", 1000), (FWD, "SQ_VALU_MFMA_BUSY_CYCLES", 2680),
+                                       (FWD, "SQ_WAIT_INST_LDS", 400), ("at::native::fill", "SQ_WAVE_CYCLES", 5)]):
+            fh.write(f'{i},"{k}",{c},{v}\n')
+    with open(tcc, "w") as fh:
+        fh.write(HEADER)
+        for i, (k, c, v) in enumerate([(FWD, "TCC_HIT_sum", 750), (FWD, "TCC_MISS_sum", 250)]):
+            fh.write(f'{i},"{k}",{c},{v}\n')
+    res = subprocess.run([sys.executable, "-m", "mindspeed_amd.profile_tools", "counters", str(sq), str(tcc)],
+                         cwd=ROOT, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+    assert "at::native" not in res.stdout
+    derived = [l for l in res.stdout.split("# derived")[1].splitlines() if l.startswith("gmm16_fast_kernel")][0].split()
+    assert derived[-5:] == ["0.670", "0.100", "-", "-", "0.750"]
+
+
+def test_products_reads_the_dispatches_in_launch_order(tmp_path):
+    """Six products, two launches each, the first of each left out: 128-byte read requests, 64-byte write requests."""
+    path = tmp_path / "c.csv"
+    with open(path, "w") as fh:
+        fh.write(HEADER)
+        d = 0
+        for prod in range(6):
+            for rep in range(2):
+                for c, v in (("TCC_EA0_RDREQ_sum", (prod + 1) * 1e7 * (3 if rep == 0 else 1)), ("TCC_EA0_WRREQ_sum", 1e7),
+                             ("TCC_HIT_sum", 3e6), ("TCC_MISS_sum", 1e6)):
+                    fh.write(f'{d},"{DW if prod > 3 else FWD}",{c},{v}\n')
+                d += 1
+    res = subprocess.run([sys.executable, "-m", "mindspeed_amd.profile_tools", "products", "--csv", str(path), "--iters", "2"],
+                         cwd=ROOT, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+    rows = {l.split()[0]: l.split()[1:] for l in res.stdout.splitlines()[1:]}
+    assert rows["fwd1"] == ["1.28", "0.64", "0.750"] and rows["dw2"] == ["7.68", "0.64", "0.750"]
+    res = subprocess.run([sys.executable, "-m", "mindspeed_amd.profile_tools", "products", "--csv", str(path), "--iters", "3"],
+                         cwd=ROOT, capture_output=True, text=True)
+    assert res.returncode != 0 and "expected 18" in res.stderr
+
+
+def test_in_layer_durations_are_recorded_with_the_build(tmp_path):
+    stats, out = tmp_path / "s.csv", tmp_path / "in_layer.json"
+    with open(stats, "w") as fh:
+        fh.write('"Name","Calls","TotalDurationNs","AverageNs","Percentage","MinNs","MaxNs","StdDev"\n')
+        fh.write('"void ms::(anonymous namespace)::permute_fused_kernel<long, unsigned int __vector(4)>(int)",50,1000000,20000.0,1,1,1,1\n')
+        fh.write('"void ms::(anonymous namespace)::swiglu_kernel<ms::BF16, 8>(int)",50,5000000,100000.0,1,1,1,1\n')
+        fh.write('"void ms::(anonymous namespace)::gmm16_fast_kernel<0, true, false, 0, true>(ms::GmmArgs)",100,1,1300000.0,1,1,1,1\n')
+    res = subprocess.run([sys.executable, "-m", "mindspeed_amd.profile_tools", "in-layer", "--stats", str(stats), "--out", str(out)],
+                         cwd=ROOT, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+    data = json.loads(out.read_text())
+    assert data["build"] == build.source_hash()
+    k = data["kernels"]["mixtral"]
+    assert set(k) == {"permute_fused_kernel", "swiglu_kernel"}
+    # 100,794,368 bytes in 20 us = 5039.7 GB/s = 0.63 of 8 TB/s
+    assert k["permute_fused_kernel"]["bytes_per_launch"] == 100794368 and k["permute_fused_kernel"]["frac_of_hbm_peak"] == 0.63
+    sys.path.insert(0, ROOT)
+    import bench
+    saved = bench.IN_LAYER_FILE
+    try:
+        bench.IN_LAYER_FILE = str(out)
+        assert bench.measured_in_layer_durations("mixtral") == k
+        data["build"] = "0" * 16
+        out.write_text(json.dumps(data))
+        assert bench.measured_in_layer_durations("mixtral") is None       # measured on other sources: not reported
+    finally:
+        bench.IN_LAYER_FILE = saved
