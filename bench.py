@@ -454,7 +454,7 @@ def main():
                     "over the average, against the 8 TB/s HBM peak and against the plain copy kernel in the same mode",
             "cold_buffer_sets": cold_sets, "warm": warm, "cold": cold}
         if args.workload == "mixtral":
-            # the same at the shapes of the other two BASELINE configurations (index form and routing-map form of the
+            # the same at the shapes of the other two benchmark configurations (index form and routing-map form of the
             # four ops, and the copy), fraction of the 8 TB/s peak and of the copy: their buffers exceed the
             # last-level cache already with one set, the rotation ("cold") adds a second or third
             brief = ("permute", "permute_mask", "unpermute", "unpermute_mask", "unpermute_grad", "permute_grad", "copy")

@@ -1,4 +1,4 @@
-"""GPU parity at BASELINE.json's full sizes: the Mixtral-shape layer (forward + backward), the DeepSeek-V3-style
+"""GPU parity at the benchmark configurations' full sizes: the Mixtral-shape layer (forward + backward), the DeepSeek-V3-style
 local share (Zipf routing with one empty expert) and the fine-grained Qwen-MoE-like layer (64 experts, top-8).
 
 Inputs come from the benchmark's own recipe (mindspeed_amd.workloads), so what is timed is what is checked.
