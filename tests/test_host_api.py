@@ -265,6 +265,54 @@ def test_shapes_propagate_on_meta_tensors():
     assert xc.grad.shape == (T, H) and pc.grad.shape == (T,)
 
 
+def test_caller_side_modules_run_on_meta_tensors():
+    """The expert module (one-node and op-by-op bodies, with activation recomputation), ``BF16GMMFunction`` and the fused
+    chunk sort's own names carry shapes and gradients on meta tensors: no device is needed to trace them."""
+    import types
+
+    import torch.nn.functional as F
+
+    from mindspeed_amd.experts import GroupedMLP
+    from mindspeed_amd.grouped_matmul_util import BF16GMMFunction, get_gmm_op_cls
+    from mindspeed_amd.ops import sort_chunks as SC
+
+    def meta(*shape, dtype=torch.bfloat16, grad=False):
+        return torch.empty(*shape, dtype=dtype, device="meta", requires_grad=grad)
+
+    E, H, FF, R = 4, 64, 32, 100
+    tpe = torch.tensor([25, 25, 25, 25])
+    for fuse in (True, False):
+        for recompute in (False, True):
+            cfg = types.SimpleNamespace(hidden_size=H, moe_ffn_hidden_size=FF, gated_linear_unit=True,
+                                        activation_func=F.silu, params_dtype=torch.bfloat16, device="meta",
+                                        moe_fuse_expert_mlp=fuse, recompute_activation_function=recompute)
+            mlp = GroupedMLP(E, cfg)
+            mlp.layer_number = 1
+            assert mlp.weight1.shape == (H, E * 2 * FF) and mlp.weight2.shape == (E * FF, H)
+            x, probs = meta(R, H, grad=True), meta(R, grad=True)
+            out, bias = mlp(x, tpe, probs)
+            assert out.shape == (R, H) and out.dtype == torch.bfloat16 and bias is None
+            out.sum().backward()
+            assert x.grad.shape == x.shape and probs.grad.shape == probs.shape
+            assert mlp.weight1.grad.shape == mlp.weight1.shape and mlp.weight2.grad.shape == mlp.weight2.shape
+
+    assert get_gmm_op_cls() is BF16GMMFunction
+    x, w, gl = meta(R, H, grad=True), meta(E, H, 2 * FF, grad=True), meta(E, dtype=torch.int64)
+    y = BF16GMMFunction.apply(x, w, None, gl, 0)
+    assert y.shape == (R, 2 * FF)
+    y.sum().backward()
+    assert x.grad.shape == x.shape and w.grad.shape == w.shape
+
+    with pytest.raises(AssertionError):                  # the fused form takes device tensors only
+        SC.moe_sort_chunks_by_index(torch.zeros(8, 4), torch.tensor([4, 4]), torch.tensor([1, 0]))
+    xc, pc = meta(R, H, grad=True), meta(R, dtype=torch.float32, grad=True)
+    sizes, order = meta(4, dtype=torch.int64), meta(4, dtype=torch.int64)
+    assert SC.moe_sort_chunks_by_index(xc, sizes, order).shape == (R, H)
+    oc, opc = SC.moe_sort_chunks_by_index_with_probs(xc, pc, sizes, order)
+    (oc.sum() + opc.sum()).backward()
+    assert xc.grad.shape == (R, H) and pc.grad.shape == (R,)
+
+
 def test_trace_and_microbench_builds_are_wired():
     """The diagnostic (tile trace) build and the measurement helpers have output paths of their own, and the plain copy
     kernel is not part of the product's C ABI."""
