@@ -265,6 +265,9 @@ _define("swiglu_grad(Tensor grad_y, Tensor x, Tensor? probs) -> (Tensor, Tensor)
 
 
 # ---- routing-map (mask) form ---------------------------------------------------------------------------------
+_ROUTING_MAP_WS = {}     # workspace bytes by (tokens, experts, mode): the size query is pure host arithmetic
+
+
 def _routing_map_permute(tokens, routing_map, num_rows, drop_and_pad, want_counts):
     """``tokens`` may be None (maps only).  Returns (permuted or empty, row_id_map, sorted_flat, counts or empty)."""
     lib = _lib.load()
@@ -281,10 +284,16 @@ def _routing_map_permute(tokens, routing_map, num_rows, drop_and_pad, want_count
         permuted = torch.empty((num_rows, hidden), dtype=tokens.dtype, device=dev)
     else:
         permuted = torch.empty(0, dtype=torch.float32, device=dev)
-    nbytes = ctypes.c_size_t(0)
-    _lib.check(lib.ms_moe_routing_map_workspace_size(num_tokens, num_experts, int(drop_and_pad), ctypes.byref(nbytes)),
-               "ms_moe_routing_map_workspace_size")
-    ws = _lib.workspace(nbytes.value, dev)
+    key = (num_tokens, num_experts, bool(drop_and_pad))
+    need = _ROUTING_MAP_WS.get(key)
+    if need is None:
+        nbytes = ctypes.c_size_t(0)
+        _lib.check(lib.ms_moe_routing_map_workspace_size(num_tokens, num_experts, int(drop_and_pad),
+                                                         ctypes.byref(nbytes)), "ms_moe_routing_map_workspace_size")
+        if len(_ROUTING_MAP_WS) > 4096:
+            _ROUTING_MAP_WS.clear()
+        need = _ROUTING_MAP_WS[key] = nbytes.value
+    ws = _lib.workspace(need, dev)
     work = (num_tokens * hidden * elem + num_rows * hidden * elem if tokens is not None else 0) \
         + num_tokens * num_experts * (1 + 4) + num_rows * 4
     with _lib.on(dev), flop_counter.op("permute", work, "byte", dev):
