@@ -145,14 +145,19 @@ def cpu_baseline(cfg, budget_s=12.0):
         w1 = torch.randn(1, H, 2 * F // 8, generator=gen).mul_(0.02).repeat(E, 1, 8)
         w2 = torch.randn(1, F // 8, H, generator=gen).mul_(0.02).repeat(E, 8, 1)
         pw, idxw = make_routing(cfg, 0)
+        times = []
         with torch.no_grad():
-            t0 = time.perf_counter()
-            O.moe_layer(xw, idxw, pw.float(), w1, w2)
-            dtw = time.perf_counter() - t0
+            for _ in range(5):
+                t0 = time.perf_counter()
+                O.moe_layer(xw, idxw, pw.float(), w1, w2)
+                times.append(time.perf_counter() - t0)
+                if sum(times) > 25.0:          # a slow host: what has been run so far has to do
+                    break
         del xw, w1, w2
+        dtw = sorted(times)[len(times) // 2]
         extra["whole_forward"] = {"value": round(T / dtw, 1), "unit": "tokens/s", "cores": threads,
-                                  "sample": f"all {T} tokens of the workload, forward pass only (configs[1]), fp32, one "
-                                            f"run ({dtw:.1f} s): no extrapolation"}
+                                  "sample": f"all {T} tokens of the workload, forward pass only (configs[1]), fp32, "
+                                            f"median of {len(times)} runs ({dtw:.1f} s): no extrapolation"}
     # configs[0], the reference's CPU-runnable case, whole (no extrapolation): median of five runs
     from mindspeed_amd.workloads import WORKLOADS
     small = WORKLOADS["plumbing"]
