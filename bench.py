@@ -14,6 +14,7 @@ accumulation).  One JSON line is printed.
 from __future__ import annotations
 
 import argparse
+import contextlib
 import json
 import os
 import sys
@@ -174,7 +175,37 @@ def cpu_baseline(cfg, budget_s=12.0):
             "cpu_model": _cpu_model(), "host_cores": os.cpu_count()}
 
 
-def measure_routing_map_mode(cfg, device, x, idx, p, iters=20, warmup=5):
+@contextlib.contextmanager
+def threads_on_one_core():
+    """Confine every thread of this process to one core for the duration.  The host work of an eager step is serial —
+    the main thread issues the forward pass, then waits while torch's autograd thread issues the backward pass — so
+    nothing is lost, and the core never goes idle between the two hand-overs of a step.  With the threads on different
+    cores each hand-over wakes an idle core, which on these hosts costs about 70 us: the small configuration's step
+    reads 0.43-0.45 ms that way and 0.29-0.32 ms on one core (whichever placement the scheduler picks decides the
+    figure otherwise: runs of the same loop switch between the two)."""
+    saved = {}
+    for name in os.listdir("/proc/self/task"):
+        try:
+            saved[int(name)] = os.sched_getaffinity(int(name))
+        except OSError:
+            pass
+    core = {min(os.sched_getaffinity(0))}
+    try:
+        for tid in saved:
+            try:
+                os.sched_setaffinity(tid, core)
+            except OSError:
+                pass
+        yield
+    finally:
+        for tid, mask in saved.items():
+            try:
+                os.sched_setaffinity(tid, mask)
+            except OSError:
+                pass
+
+
+def measure_routing_map_mode(cfg, device, x, idx, p, iters=200, warmup=20):
     """The routing-map (mask) form of permute / unpermute on the same workload: event-timed averages of the
     forward and of forward+backward, with the algorithmic bytes of the row movement.  Not part of `value`."""
     from mindspeed_amd.ops import moe_permute_mask_map as M
@@ -492,6 +523,13 @@ def main():
                         "gemm_tflops": {k: ok[k]["tflops"] for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok},
                         "gemm_frac_of_mfma_peak": {k: ok[k]["frac_of_mfma_peak"]
                                                    for k in ("gmm_fwd", "gmm_dx", "gmm_dw") if k in ok}}
+        if small:
+            # the same steps with the process's threads on one core (see threads_on_one_core)
+            with threads_on_one_core():
+                ms1, _, _, _ = run_layer(ocfg, device, steps=300, warmup=100, per_kernel=False)
+            others[name]["ms_per_step_threads_on_one_core"] = round(ms1, 4)
+            others[name]["note"] = ("ms_per_step: threads placed by the scheduler; the step is host-bound and reads "
+                                    "0.27-0.45 ms depending on whether the main and the autograd thread share a core")
 
     def graph_section():
         others["plumbing"]["graph_replay_ms_per_step"] = graph_replay_ms(WORKLOADS["plumbing"], device)
