@@ -470,6 +470,11 @@ def main():
 
     def routing_map_section():
         result["routing_map_mode"] = measure_routing_map_mode(cfg, device, x.detach(), idx, p.detach())
+        # these loops are host-bound too, and the forward+backward ones hand over to the autograd thread
+        with threads_on_one_core():
+            pinned = measure_routing_map_mode(cfg, device, x.detach(), idx, p.detach())
+        result["routing_map_mode"]["avg_ms_threads_on_one_core"] = {
+            k: v["avg_ms"] for k, v in pinned.items() if isinstance(v, dict)}
 
     def permute_family_section():
         # The permute / unpermute family by itself at this workload's shape: back-to-back launches through the C ABI
