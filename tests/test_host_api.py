@@ -313,6 +313,40 @@ def test_caller_side_modules_run_on_meta_tensors():
     assert xc.grad.shape == (R, H) and pc.grad.shape == (R,)
 
 
+def test_deferred_weight_gradient_queue_on_meta_tensors():
+    """``WeightGradStore`` in decoupled mode: backward returns dX only and parks the weight-gradient operands; ``pop``
+    runs the parked product later and adds it to ``main_grad``; ``clear`` resets the switch
+    (fb_overlap/modules/weight_grad_store.py:29-58,86-108)."""
+    from mindspeed_amd.grouped_matmul_util import BF16GMMFunction, WeightGradStore, gmm_settings
+
+    def meta(*shape, dtype=torch.bfloat16, grad=False):
+        return torch.empty(*shape, dtype=dtype, device="meta", requires_grad=grad)
+
+    E, H, N, R = 4, 64, 48, 100
+    x, w = meta(R, H, grad=True), torch.nn.Parameter(meta(E, H, N))
+    w.main_grad = meta(E, H, N, dtype=torch.float32)
+    gl = meta(E, dtype=torch.int64)
+    WeightGradStore.clear()
+    try:
+        WeightGradStore.is_decoupleBlock = True
+        y = BF16GMMFunction.apply(x, w, None, gl, w)
+        y.sum().backward()
+        assert x.grad.shape == x.shape and w.grad is None          # dW was not computed in backward
+        assert len(WeightGradStore.cache) == 1
+        (ctx_and_inputs, grad_output, weight_param, _sp, _in_row) = WeightGradStore.cache[0]
+        assert weight_param is w and grad_output.shape == (R, N) and ctx_and_inputs[1].shape == (R, H)
+        for fusion in (False, True):
+            gmm_settings.gemm_gradient_accumulation_fusion = fusion
+            if fusion:                                                 # park the same operands once more
+                WeightGradStore.put(ctx_and_inputs, grad_output, weight_param)
+            WeightGradStore.pop()
+            assert not WeightGradStore.cache and w.main_grad.shape == (E, H, N)
+    finally:
+        gmm_settings.gemm_gradient_accumulation_fusion = False
+        WeightGradStore.clear()
+    assert WeightGradStore.is_decoupleBlock is False and WeightGradStore.cache == []
+
+
 def test_trace_and_microbench_builds_are_wired():
     """The diagnostic (tile trace) build and the measurement helpers have output paths of their own, and the plain copy
     kernel is not part of the product's C ABI."""
